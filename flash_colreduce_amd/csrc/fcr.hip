@@ -1,0 +1,523 @@
+// libfcr: column reduction of softmax attention for MI355X (gfx950, CDNA4).
+//
+// Two kernels, both built on v_mfma_f32_32x32x16_{f16,bf16} with the product taken as
+// S^T = K * Q^T (keys are MFMA rows, queries are MFMA columns).  In the 32x32 accumulator a lane
+// owns ONE query (lane & 31) and 16 keys (row 8*(r/4) + 4*(lane/32) + r%4 for register r), so
+//   - everything that is per query row (softmax reference exponent, running sum, lse) is one
+//     scalar per lane and needs no cross-lane traffic inside the sweep;
+//   - everything that is per key column accumulates in the lane's 16 registers over the whole
+//     sweep and is reduced across the 32 query lanes once, at the end.
+//
+//   row_lse_kernel    a workgroup keeps 256 query rows in registers (64 per wave) and streams
+//                     key tiles through LDS; writes lse2[bh, i] = log2 sum_j 2^(s_ij).
+//   col_reduce_kernel a workgroup keeps 256 key rows in registers and streams query tiles (and
+//                     their lse2) through LDS; writes out[bh, j] = sum_i or max_i 2^(s_ij-lse2_i).
+// where s_ij = scale * log2(e) * <q_i, k_j>.  Nothing of size M*N is written anywhere and there
+// are no atomics: one workgroup owns its output rows / columns.
+//
+// Replaces the Triton kernel of the reference (flash_colreduce/flash.py:11-274).
+
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "fcr.h"
+
+namespace {
+
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int kWaves = 4;
+constexpr int kThreads = kWaves * 64;
+constexpr int kWaveRows = 64;                 // resident rows per wave: two 32-row MFMA blocks
+constexpr int kTileRows = kWaves * kWaveRows; // resident rows per workgroup
+constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row blocks)
+constexpr float kNegInf = -__builtin_inff();
+constexpr float kPosInf = __builtin_inff();
+
+struct Params {
+  const char* q;
+  const char* k;
+  float* lse;        // [BH, M]
+  float* out;        // [BH, N]
+  int64_t q_sb, q_sh, q_sr;  // strides in BYTES: batch, head, row
+  int64_t k_sb, k_sh, k_sr;
+  int H, M, N;
+  int dgran;         // D / 8: valid 16-byte granules per row
+  int c;             // max(N - M, 0): the causal right-alignment offset
+  float scale2;      // scale * log2(e)
+  int tiles;         // resident tiles per (b,h)
+  int total;         // tiles * B * H
+};
+
+template <int DT>
+__device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
+  if constexpr (DT == FCR_DTYPE_F16) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
+                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+  } else {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
+                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+  }
+}
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// Key offset inside a 32-row block of accumulator register r, before the 4*(lane/32) term.
+__device__ __forceinline__ constexpr int reg_row(int r) { return 8 * (r >> 2) + (r & 3); }
+
+// Workgroups are dealt to the 8 XCDs round-robin by blockIdx.  Give each XCD a contiguous run
+// of (b,h) so that the streamed operand of a head stays in one XCD's L2, and inside a head hand
+// out the tiles with the longest sweep first.
+__device__ __forceinline__ bool map_block(const Params& p, bool reverse, int& bh, int& tile) {
+  const int per = (p.total + 7) >> 3;
+  const int v = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
+  if (v >= p.total) return false;
+  bh = v / p.tiles;
+  const int t = v - bh * p.tiles;
+  tile = reverse ? p.tiles - 1 - t : t;
+  return true;
+}
+
+// The operand a wave keeps for the whole sweep: rows [row0, row0+64), as MFMA fragments.
+// Lane l holds, for k-step ks, the 8 elements [16*ks + 8*(l/32), +8) of row (l & 31) of a block.
+template <int KS>
+__device__ __forceinline__ void load_resident(u32x4 (&f)[2][KS], const char* base, int64_t row_bytes,
+                                              int row0, int nrows, int dgran, int lane) {
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    const int row = row0 + blk * 32 + (lane & 31);
+    const char* src = base + (int64_t)row * row_bytes;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int g = ks * 2 + (lane >> 5);
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (row < nrows && g < dgran) v = *reinterpret_cast<const u32x4*>(src + g * 16);
+      f[blk][ks] = v;
+    }
+  }
+}
+
+// Global -> registers -> LDS staging of kChunk rows of the streamed operand.
+// LDS rows are padded by 16 bytes so that the 16-byte fragment reads of 16 consecutive rows
+// fall into distinct banks.
+template <int KS>
+struct Stager {
+  static constexpr int kGran = 2 * KS;             // 16-byte granules per (zero padded) row
+  static constexpr int kRowBytes = KS * 32 + 16;   // LDS row pitch
+  static constexpr int kTotal = kChunk * kGran;
+  static constexpr int kPer = (kTotal + kThreads - 1) / kThreads;
+  static constexpr int kBytes = kChunk * kRowBytes;
+  u32x4 regs[kPer];
+
+  __device__ __forceinline__ void load(const char* base, int64_t row_bytes, int row0, int nrows,
+                                       int dgran, int tid) {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int g = tid + i * kThreads;
+      const int r = g / kGran, cg = g - r * kGran;
+      const int row = row0 + r;
+      u32x4 v = {0u, 0u, 0u, 0u};
+      if (g < kTotal && row < nrows && cg < dgran)
+        v = *reinterpret_cast<const u32x4*>(base + (int64_t)row * row_bytes + cg * 16);
+      regs[i] = v;
+    }
+  }
+  __device__ __forceinline__ void store(char* lds, int tid) const {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int g = tid + i * kThreads;
+      const int r = g / kGran, cg = g - r * kGran;
+      if (g < kTotal) *reinterpret_cast<u32x4*>(lds + r * kRowBytes + cg * 16) = regs[i];
+    }
+  }
+  // Fragment of block `sub` (32 rows) for k-step ks.
+  static __device__ __forceinline__ u32x4 frag(const char* lds, int sub, int ks, int lane) {
+    return *reinterpret_cast<const u32x4*>(lds + (sub * 32 + (lane & 31)) * kRowBytes + ks * 32 +
+                                           (lane >> 5) * 16);
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// Row statistics.  Per lane and 32-query block the state is (mref, l) with
+//   sum over the keys seen so far of 2^(s) = l * 2^mref.
+// mref is a reference exponent, not the running maximum: the common path adds 2^(s - mref)
+// without looking for a maximum.  The sum is renormalised only when it leaves [1, 2^64) -- the
+// first visible keys of a row, or a jump of the scores by more than 64 binades -- and then
+// exactly as the classic online softmax would (new reference = old + max(tile max, 0)).
+// Invariant after the first visible key: 1 <= l < 2^64, hence mref <= lse < mref + 64, so terms
+// that underflow are below 2^-126 of the total and overflow is caught by the range check.
+template <bool MASK>
+__device__ __forceinline__ void lse_update(const f32x16& acc, float scale2, float& mref, float& l,
+                                           int lim) {
+  const float nm = -mref;
+  float t[16];
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float x = fmaf(acc[r], scale2, nm);
+    if (MASK) x = (reg_row(r) <= lim) ? x : kNegInf;
+    t[r] = x;
+    if (r & 1) s1 += fast_exp2(x); else s0 += fast_exp2(x);
+  }
+  const float ln = l + (s0 + s1);
+  const bool ok = (ln >= 1.0f) && (ln < 1.8446744e19f);
+  if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+    l = ln;
+    return;
+  }
+  float tmax = t[0];
+#pragma unroll
+  for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, t[r]);
+  float delta;
+  if (l == 0.f) delta = (tmax > kNegInf) ? tmax : 0.f;
+  else delta = fmaxf(tmax, 0.f);
+  float s = 0.f;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) s += fast_exp2(t[r] - delta);
+  l = l * fast_exp2(-delta) + s;
+  mref += delta;
+}
+
+__device__ __forceinline__ float lse_merge(float a, float b) {
+  const float hi = fmaxf(a, b), lo = fminf(a, b);
+  if (hi == kNegInf) return kNegInf;
+  return hi + fast_log2(1.0f + fast_exp2(lo - hi));
+}
+
+template <int DT, int KS, bool CAUSAL>
+__global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
+  using St = Stager<KS>;
+  __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
+  int bh, tile;
+  if (!map_block(p, CAUSAL, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = bh / p.H, h = bh - b * p.H;
+  const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+  const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
+
+  const int q0 = tile * kTileRows + wave * kWaveRows;  // first query of this wave
+  u32x4 qf[2][KS];
+  load_resident<KS>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
+
+  // keys this workgroup / this wave has to look at
+  const int kend_wg = CAUSAL ? min(p.N, tile * kTileRows + kTileRows + p.c) : p.N;
+  const int nchunks = (kend_wg + kChunk - 1) / kChunk;
+
+  float mref[2] = {0.f, 0.f}, l[2] = {0.f, 0.f};
+  // last key a lane's query may see, per block
+  int last[2];
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    const int i = q0 + blk * 32 + (lane & 31);
+    last[blk] = (CAUSAL ? min(p.N - 1, i + p.c) : p.N - 1) - 4 * (lane >> 5);
+  }
+
+  St st;
+  st.load(kb, p.k_sr, 0, p.N, p.dgran, tid);
+  int buf = 0;
+  for (int t = 0; t < nchunks; ++t) {
+    char* lds = smem + buf * St::kBytes;
+    st.store(lds, tid);
+    __syncthreads();
+    if (t + 1 < nchunks) st.load(kb, p.k_sr, (t + 1) * kChunk, p.N, p.dgran, tid);
+#pragma unroll
+    for (int sub = 0; sub < kChunk / 32; ++sub) {
+      const int key0 = t * kChunk + sub * 32;
+      if (key0 >= p.N) continue;
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        const int qblk = q0 + blk * 32;
+        if (CAUSAL && key0 > qblk + 31 + p.c) continue;  // block cannot see this sub-tile
+        f32x16 acc = {0};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) acc = mma<DT>(St::frag(lds, sub, ks, lane), qf[blk][ks], acc);
+        const bool need_mask = (key0 + 32 > p.N) || (CAUSAL && key0 + 31 > qblk + p.c);
+        if (need_mask) lse_update<true>(acc, p.scale2, mref[blk], l[blk], last[blk] - key0);
+        else lse_update<false>(acc, p.scale2, mref[blk], l[blk], 0);
+      }
+    }
+    buf ^= 1;
+  }
+
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk) {
+    float v = (l[blk] > 0.f) ? mref[blk] + fast_log2(l[blk]) : kNegInf;
+    const float o = __shfl_xor(v, 32);
+    v = lse_merge(v, o);
+    const int i = q0 + blk * 32 + lane;
+    if (lane < 32 && i < p.M) p.lse[(int64_t)bh * p.M + i] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+template <bool MASK, bool ISMAX>
+__device__ __forceinline__ void col_update(const f32x16& acc, float scale2, float nlse, f32x16& col,
+                                           int lim) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float x = fmaf(acc[r], scale2, nlse);
+    if (MASK) x = (reg_row(r) <= lim) ? x : kNegInf;
+    if (ISMAX) col[r] = fmaxf(col[r], x);
+    else col[r] += fast_exp2(x);
+  }
+}
+
+template <int DT, int KS, bool CAUSAL, bool ISMAX>
+__global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p) {
+  using St = Stager<KS>;
+  constexpr int kStage = St::kBytes + kChunk * 4;     // rows + their lse
+  constexpr int kRed = kWaves * 32 * 64 * 4;          // end-of-sweep transpose buffer
+  constexpr int kSmem = (2 * kStage > kRed) ? 2 * kStage : kRed;
+  __shared__ __attribute__((aligned(16))) char smem[kSmem];
+  int bh, tile;
+  if (!map_block(p, false, bh, tile)) return;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int b = bh / p.H, h = bh - b * p.H;
+  const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+  const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
+  const float* lse = p.lse + (int64_t)bh * p.M;
+
+  const int k0 = tile * kTileRows + wave * kWaveRows;  // first key of this wave
+  u32x4 kf[2][KS];
+  load_resident<KS>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
+
+  f32x16 col[2];
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) col[blk][r] = ISMAX ? kNegInf : 0.f;
+
+  // first query chunk that can see any key of this tile
+  const int t0 = CAUSAL ? max(0, tile * kTileRows - p.c) / kChunk : 0;
+  const int nchunks = (p.M + kChunk - 1) / kChunk;
+  // lim = i + c - key0(blk) - 4*(lane/32), with i the lane's query in the current sub-tile
+  const int lim_lane = (lane & 31) + p.c - 4 * (lane >> 5);
+
+  St st;
+  float lse_reg = kPosInf;
+  auto load_lse = [&](int row0) {
+    if (tid < kChunk) {
+      const int i = row0 + tid;
+      lse_reg = (i < p.M) ? lse[i] : kPosInf;  // +inf: rows past M contribute 2^-inf = 0
+    }
+  };
+  if (t0 < nchunks) {
+    st.load(qb, p.q_sr, t0 * kChunk, p.M, p.dgran, tid);
+    load_lse(t0 * kChunk);
+  }
+  int buf = 0;
+  for (int t = t0; t < nchunks; ++t) {
+    char* lds = smem + buf * kStage;
+    float* lds_lse = reinterpret_cast<float*>(lds + St::kBytes);
+    st.store(lds, tid);
+    if (tid < kChunk) lds_lse[tid] = lse_reg;
+    __syncthreads();
+    if (t + 1 < nchunks) {
+      st.load(qb, p.q_sr, (t + 1) * kChunk, p.M, p.dgran, tid);
+      load_lse((t + 1) * kChunk);
+    }
+#pragma unroll
+    for (int sub = 0; sub < kChunk / 32; ++sub) {
+      const int qs = t * kChunk + sub * 32;  // first query of the sub-tile
+      if (qs >= p.M) continue;
+      const float nlse = -lds_lse[sub * 32 + (lane & 31)];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        const int kblk = k0 + blk * 32;
+        if (kblk >= p.N) continue;
+        if (CAUSAL && kblk > qs + 31 + p.c) continue;  // no query of the sub-tile sees this block
+        f32x16 acc = {0};
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) acc = mma<DT>(kf[blk][ks], St::frag(lds, sub, ks, lane), acc);
+        const bool need_mask = CAUSAL && (kblk + 31 > qs + p.c);
+        if (need_mask) col_update<true, ISMAX>(acc, p.scale2, nlse, col[blk], lim_lane + qs - kblk);
+        else col_update<false, ISMAX>(acc, p.scale2, nlse, col[blk], 0);
+      }
+    }
+    buf ^= 1;
+  }
+
+  // Reduce over the 32 query lanes: transpose through LDS, one output key per lane.
+  __syncthreads();
+  float* red = reinterpret_cast<float*>(smem) + wave * (32 * 64);
+#pragma unroll
+  for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) red[(blk * 16 + r) * 64 + lane] = col[blk][r];
+  __syncthreads();
+  {
+    const int w = lane & 31;
+    const int idx = (lane >> 5) * 16 + (w >> 3) * 4 + (w & 3);
+    const float* src = red + idx * 64 + ((w >> 2) & 1) * 32;
+    float v = ISMAX ? kNegInf : 0.f;
+#pragma unroll 8
+    for (int j = 0; j < 32; ++j) {
+      const float x = src[(j + lane) & 31];
+      v = ISMAX ? fmaxf(v, x) : v + x;
+    }
+    if (ISMAX) v = fast_exp2(v);
+    const int key = k0 + lane;
+    if (key < p.N) p.out[(int64_t)bh * p.N + key] = v;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
+thread_local char g_err[256] = "";
+
+int fail(int code, const char* what) {
+  snprintf(g_err, sizeof(g_err), "%s", what);
+  return code;
+}
+
+int check_strides(const void* ptr, const int64_t s[4], const char* name) {
+  if (s[3] != 1) {
+    snprintf(g_err, sizeof(g_err), "%s: stride of the last dimension must be 1 (got %lld)", name, (long long)s[3]);
+    return FCR_E_STRIDE;
+  }
+  if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0 || s[0] % 8 != 0 || s[1] % 8 != 0 || s[2] % 8 != 0 ||
+      s[0] < 0 || s[1] < 0 || s[2] < 0) {
+    snprintf(g_err, sizeof(g_err),
+             "%s: base pointer must be 16-byte aligned and batch/head/row strides non-negative multiples of 8 elements",
+             name);
+    return FCR_E_STRIDE;
+  }
+  return 0;
+}
+
+int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H, int M, int N, int D,
+                const int64_t qs[4], const int64_t ks[4], float scale, bool by_keys) {
+  if (!q || !k || !qs || !ks) return fail(FCR_E_NULL, "null pointer argument");
+  if (dtype != FCR_DTYPE_F16 && dtype != FCR_DTYPE_BF16) return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16 or FCR_DTYPE_BF16");
+  if (B < 1 || H < 1 || M < 1 || N < 1) return fail(FCR_E_SHAPE, "B, H, M, N must be >= 1");
+  if (D < 8 || D > 128 || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 128]");
+  if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
+  const int64_t bh = (int64_t)B * H;
+  const int64_t tiles = ((by_keys ? N : M) + kTileRows - 1) / kTileRows;
+  if (bh * tiles > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
+  if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
+  int rc = check_strides(q, qs, "q");
+  if (rc) return rc;
+  rc = check_strides(k, ks, "k");
+  if (rc) return rc;
+  p.q = static_cast<const char*>(q);
+  p.k = static_cast<const char*>(k);
+  p.q_sb = qs[0] * 2; p.q_sh = qs[1] * 2; p.q_sr = qs[2] * 2;
+  p.k_sb = ks[0] * 2; p.k_sh = ks[1] * 2; p.k_sr = ks[2] * 2;
+  p.H = H; p.M = M; p.N = N;
+  p.dgran = D / 8;
+  p.c = N > M ? N - M : 0;
+  p.scale2 = (float)((double)scale * 1.4426950408889634);
+  p.tiles = (int)tiles;
+  p.total = (int)(bh * tiles);
+  p.lse = nullptr;
+  p.out = nullptr;
+  return 0;
+}
+
+int launched(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e == hipSuccess) return 0;
+  snprintf(g_err, sizeof(g_err), "%s launch failed: %s", what, hipGetErrorString(e));
+  return (int)e;
+}
+
+template <int DT, int KS>
+void launch_lse(const Params& p, bool causal, hipStream_t s) {
+  const dim3 grid(((p.total + 7) / 8) * 8), block(kThreads);
+  if (causal) hipLaunchKernelGGL((row_lse_kernel<DT, KS, true>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((row_lse_kernel<DT, KS, false>), grid, block, 0, s, p);
+}
+
+template <int DT, int KS>
+void launch_col(const Params& p, bool causal, bool ismax, hipStream_t s) {
+  const dim3 grid(((p.total + 7) / 8) * 8), block(kThreads);
+  if (causal) {
+    if (ismax) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, true>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, false>), grid, block, 0, s, p);
+  } else {
+    if (ismax) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, true>), grid, block, 0, s, p);
+    else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, false>), grid, block, 0, s, p);
+  }
+}
+
+#define FCR_DISPATCH_KS(DT, ksteps, CALL)                  \
+  switch (ksteps) {                                        \
+    case 1: CALL(DT, 1); break;                            \
+    case 2: CALL(DT, 2); break;                            \
+    case 3: CALL(DT, 3); break;                            \
+    case 4: CALL(DT, 4); break;                            \
+    case 5: CALL(DT, 5); break;                            \
+    case 6: CALL(DT, 6); break;                            \
+    case 7: CALL(DT, 7); break;                            \
+    default: CALL(DT, 8); break;                           \
+  }
+
+}  // namespace
+
+extern "C" {
+
+int fcr_version(void) { return FCR_VERSION; }
+
+const char* fcr_last_error(void) { return g_err; }
+
+size_t fcr_lse_bytes(int B, int H, int M) {
+  if (B < 0 || H < 0 || M < 0) return 0;
+  return (size_t)B * (size_t)H * (size_t)M * sizeof(float);
+}
+
+int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int H, int M, int N, int D,
+                const int64_t q_strides[4], const int64_t k_strides[4], float scale, int causal,
+                void* stream) {
+  Params p;
+  if (!lse) return fail(FCR_E_NULL, "null pointer argument");
+  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, false);
+  if (rc) return rc;
+  p.lse = lse;
+  const int ksteps = (D + 15) / 16;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal != 0, s)
+  if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_LSE) }
+  else { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_LSE) }
+#undef FCR_CALL_LSE
+  return launched("row_lse_kernel");
+}
+
+int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, int dtype, int B, int H,
+                   int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
+                   float scale, int reduction, int causal, void* stream) {
+  Params p;
+  if (!lse || !out) return fail(FCR_E_NULL, "null pointer argument");
+  if (reduction != FCR_REDUCE_SUM && reduction != FCR_REDUCE_MAX)
+    return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM or FCR_REDUCE_MAX");
+  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true);
+  if (rc) return rc;
+  p.lse = const_cast<float*>(lse);
+  p.out = out;
+  const int ksteps = (D + 15) / 16;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal != 0, reduction == FCR_REDUCE_MAX, s)
+  if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_COL) }
+  else { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL) }
+#undef FCR_CALL_COL
+  return launched("col_reduce_kernel");
+}
+
+int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H, int M,
+                  int N, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
+                  int reduction, int causal, void* stream) {
+  if (!out || !lse_ws) return fail(FCR_E_NULL, "null pointer argument");
+  if (reduction != FCR_REDUCE_SUM && reduction != FCR_REDUCE_MAX)
+    return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM or FCR_REDUCE_MAX");
+  int rc = fcr_row_lse(q, k, lse_ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream);
+  if (rc) return rc;
+  return fcr_col_reduce(q, k, lse_ws, out, dtype, B, H, M, N, D, q_strides, k_strides, scale, reduction,
+                        causal, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,140 @@
+"""`flash_colreduce`: the reference's operator interface on top of libfcr.so.
+
+Mirrors flash_colreduce/flash.py:311-385 (signature, validation order, error messages, default
+scale, mean epilogue, output dtype).  The device work is two hand-written gfx950 kernels behind
+a C ABI (include/fcr.h); torch is used for device memory and the current stream only.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+__all__ = ["flash_colreduce", "row_lse2"]
+
+_DTYPES = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}
+
+
+def _validate(query: torch.Tensor, key: torch.Tensor, reduction: Optional[str]):
+    # flash.py:354-364, same order and messages
+    if not query.is_cuda or not key.is_cuda:
+        raise ValueError("Query and key tensors must be on CUDA device.")
+    if query.dim() != 4 or key.dim() != 4 or not all(query.shape[i] == key.shape[i] for i in (0, 1, 3)):
+        raise ValueError(
+            f"Query and key tensors must have same batch size, number of heads, and head dimension. "
+            f"Got query shape: {query.shape}, key shape: {key.shape}."
+        )
+    if reduction is not None and reduction not in ("sum", "mean", "max"):
+        raise ValueError(f"Invalid reduction: {reduction}. Must be 'sum', 'mean', or 'max'.")
+    if query.dtype != key.dtype or query.dtype not in _DTYPES:
+        raise ValueError(
+            f"Query and key tensors must both be float16 or bfloat16. "
+            f"Got query dtype: {query.dtype}, key dtype: {key.dtype}."
+        )
+    if query.device != key.device:
+        raise ValueError("Query and key tensors must be on the same device.")
+    if query.shape[3] > 128:
+        raise ValueError(f"Head dimension must be <= 128. Got {query.shape[3]}.")
+
+
+def _device_layout(x: torch.Tensor) -> torch.Tensor:
+    """What the C ABI needs: unit d stride, 16-byte aligned rows, D a multiple of 8.
+
+    The reference pads D to a power of two (flash.py:368-373); zero columns do not change <q,k>.
+    Here a copy is made only for D % 8 != 0 or for layouts the kernels cannot address.
+    """
+    d = x.shape[3]
+    if d % 8 != 0:
+        return torch.nn.functional.pad(x, (0, 8 - d % 8))  # new contiguous tensor
+    ok = (x.stride(3) == 1 and x.data_ptr() % 16 == 0 and
+          all(x.stride(i) % 8 == 0 and x.stride(i) >= 0 for i in (0, 1, 2)))
+    return x if ok else x.contiguous()
+
+
+def _launch(query, key, reduction, is_causal, scale, want_out=True):
+    b, h, m, d = query.shape
+    n = key.shape[2]
+    if scale is None:
+        scale = 1 / math.sqrt(d)  # the unpadded D (flash.py:366-367)
+    q = _device_layout(query)
+    k = _device_layout(key)
+    lib = _lib.load()
+    dev = query.device
+    lse = torch.empty((b * h, m), device=dev, dtype=torch.float32)
+    out = torch.empty((b * h, n), device=dev, dtype=torch.float32) if want_out else None
+    if b * h * m * n == 0:
+        lse.fill_(float("-inf"))
+        if want_out:
+            out.zero_()
+    else:
+        with torch.cuda.device(dev):
+            stream = torch.cuda.current_stream(dev).cuda_stream
+            common = (_lib.DTYPE_F16 if q.dtype == torch.float16 else _lib.DTYPE_BF16,
+                      b, h, m, n, q.shape[3], _lib.strides4(q.stride()), _lib.strides4(k.stride()),
+                      float(scale))
+            if want_out:
+                red = _lib.REDUCE_MAX if reduction == "max" else _lib.REDUCE_SUM
+                _lib.check(lib.fcr_colreduce(q.data_ptr(), k.data_ptr(), out.data_ptr(), lse.data_ptr(),
+                                             *common, red, int(bool(is_causal)), stream))
+            else:
+                _lib.check(lib.fcr_row_lse(q.data_ptr(), k.data_ptr(), lse.data_ptr(), *common,
+                                           int(bool(is_causal)), stream))
+    return out, lse
+
+
+def flash_colreduce(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    reduction: str,
+    is_causal: bool = False,
+    scale: Optional[float] = None,
+    *,
+    out_dtype: Optional[torch.dtype] = None,
+) -> torch.Tensor:
+    """Per-key sum / mean / max over queries of softmax(Q K^T * scale), shape (B, H, N).
+
+    Args follow the reference (flash.py:311-352): query (B,H,M,D), key (B,H,N,D), fp16 or bf16 on
+    the GPU; `is_causal` applies the right-aligned mask (key j visible to query i iff
+    j <= i + max(N-M, 0)); `scale` defaults to 1/sqrt(D).
+
+    `out_dtype` (keyword only, not in the reference) selects the result dtype.  None reproduces
+    the reference: the fp32 accumulation is cast to query.dtype and, for 'mean', divided in that
+    dtype (flash.py:308, 377-385).  torch.float32 returns the kernel's fp32 result, with the
+    mean division done in fp32.
+    """
+    _validate(query, key, reduction)
+    b, h, m, _ = query.shape
+    n = key.shape[2]
+    res_dtype = query.dtype if out_dtype is None else out_dtype
+    if m == 0 and n > 0 and b * h > 0 and reduction == "max":
+        raise ValueError("reduction='max' needs at least one query row.")
+    if m == 0:
+        scores = torch.zeros((b, h, n), device=query.device, dtype=res_dtype)
+    else:
+        out, _ = _launch(query, key, reduction, is_causal, scale)
+        scores = out.view(b, h, n).to(res_dtype)
+    if reduction == "mean":
+        # flash.py:377-384: M for keys left of the offset, N-j from the offset on
+        if is_causal:
+            c = max(n - m, 0)
+            scores[..., :c] /= m
+            scores[..., c:] /= torch.arange(n - c, 0, -1, device=query.device)
+        else:
+            scores /= m
+    return scores
+
+
+def row_lse2(query: torch.Tensor, key: torch.Tensor, is_causal: bool = False,
+             scale: Optional[float] = None) -> torch.Tensor:
+    """Base-2 log-sum-exp of every query row over its visible keys, fp32 (B, H, M).
+
+    The hand-over between the two kernels, exposed for tests and for callers that want the
+    softmax normaliser; the reference keeps it in registers (flash.py:242).
+    """
+    _validate(query, key, None)
+    b, h, m, _ = query.shape
+    _, lse = _launch(query, key, None, is_causal, scale, want_out=False)
+    return lse.view(b, h, m)

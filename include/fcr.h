@@ -1,0 +1,100 @@
+/*
+ * fcr.h -- C ABI of libfcr.so, the MI355X (gfx950) column reduction of softmax attention.
+ *
+ * The reference has no FFI of its own: its hot path is a Python function that launches a
+ * Triton kernel (flash_colreduce/flash.py:277-308, called from flash.py:375).  These entry
+ * points are what a binding for that path has to call; each comment names the reference code
+ * the entry point stands in for.
+ *
+ * Conventions
+ *   - All pointers are DEVICE pointers on the current HIP device.  The library never
+ *     allocates, frees or keeps them.
+ *   - q is [B,H,M,D], k is [B,H,N,D], 16-bit elements (dtype below).  Strides are in ELEMENTS,
+ *     order (batch, head, row, d); the d stride must be 1, row/head/batch strides must be
+ *     multiples of 8 elements and the base pointers 16-byte aligned, D a multiple of 8 and
+ *     8 <= D <= 128.  (The reference takes any strides, flash.py:292-299; a caller with other
+ *     layouts makes a contiguous, zero-padded copy first -- the Python host does.)
+ *   - lse is fp32 [B*H, M] contiguous: per query row, log2(sum_j 2^(scale*log2(e)*<q_i,k_j>))
+ *     over the keys the row may see.  It is the hand-over between the two kernels.
+ *   - out is fp32 [B*H, N] contiguous and is fully overwritten (no zero-fill needed, unlike the
+ *     atomically accumulated buffer at flash.py:286).
+ *   - causal != 0 applies the right-aligned mask: key j takes part in row i iff
+ *     j <= i + max(N-M, 0)   (flash.py:22-27, 198-207; naive.py:20-24).
+ *   - stream is a hipStream_t (NULL = the default stream).  Launches are asynchronous.
+ *   - Return value: 0 on success; negative FCR_E_* for a rejected argument (nothing was
+ *     launched); positive = the hipError_t of a failed launch.  fcr_last_error() returns a
+ *     thread-local, human readable description of the last non-zero return on this thread.
+ *   - Thread safety: no mutable global state except the thread-local error text; calls from
+ *     several threads or streams do not interfere.
+ */
+#ifndef FCR_H
+#define FCR_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FCR_VERSION 100 /* major*10000 + minor*100 + patch */
+
+/* element type of q and k */
+#define FCR_DTYPE_F16 0
+#define FCR_DTYPE_BF16 1
+
+/* column reduction over query rows */
+#define FCR_REDUCE_SUM 0 /* also the numerator of 'mean' (flash.py:121-122) */
+#define FCR_REDUCE_MAX 1 /* flash.py:123-124 */
+
+/* argument errors */
+#define FCR_E_NULL -1      /* a required pointer is NULL */
+#define FCR_E_DTYPE -2     /* dtype is not FCR_DTYPE_* */
+#define FCR_E_SHAPE -3     /* B,H,M,N < 1, D outside [8,128] or not a multiple of 8, sizes overflow */
+#define FCR_E_STRIDE -4    /* d stride != 1 or a stride / base pointer breaks 16-byte alignment */
+#define FCR_E_REDUCTION -5 /* reduction is not FCR_REDUCE_* */
+#define FCR_E_SCALE -6     /* scale is not finite */
+
+/* Library version (FCR_VERSION it was built from). */
+int fcr_version(void);
+
+/* Text for the last non-zero return value on the calling thread ("" if none). */
+const char* fcr_last_error(void);
+
+/* Bytes of the lse hand-over buffer for a problem: B*H*M*sizeof(float). */
+size_t fcr_lse_bytes(int B, int H, int M);
+
+/*
+ * First kernel: per-row base-2 log-sum-exp over all visible keys.
+ * Stands in for the first half of the reference kernel: the two _update_softmax_lse sweeps and
+ * "lse = m + log2(l)" (flash.py:35-80, 209-242), with scale*log2(e) folded as at flash.py:291.
+ */
+int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int H, int M, int N,
+                int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
+                int causal, void* stream);
+
+/*
+ * Second kernel: out[bh, j] = reduce_i 2^(scale*log2(e)*<q_i,k_j> - lse[bh, i]) over the rows
+ * that may see key j; reduce = sum or max.  One workgroup owns a tile of key columns for the
+ * whole sweep over query rows, so there are no atomics.
+ * Stands in for the _update_softmax_cstats sweeps and their atomic_add / atomic_max
+ * (flash.py:83-126, 244-274).
+ */
+int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, int dtype, int B,
+                   int H, int M, int N, int D, const int64_t q_strides[4],
+                   const int64_t k_strides[4], float scale, int reduction, int causal,
+                   void* stream);
+
+/*
+ * Both kernels back to back on one stream: the whole of _flash_colreduce (flash.py:277-308)
+ * except the final cast to the input dtype, which stays with the host.  lse_ws is scratch of
+ * fcr_lse_bytes(B,H,M) bytes that holds the row statistics on return.
+ */
+int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H,
+                  int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
+                  float scale, int reduction, int causal, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FCR_H */

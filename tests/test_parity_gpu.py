@@ -1,0 +1,238 @@
+"""GPU parity: libfcr (through flash_colreduce / the C ABI) against the CPU oracle on the same
+seeded inputs.  Tolerances are BASELINE.json's: rtol 2e-3 / atol 1e-5 for sum and mean,
+2e-3 relative for max, checked on the kernel's fp32 result."""
+import math
+
+import pytest
+import torch
+
+import flash_colreduce_amd as fca
+from oracle.colreduce_oracle import colreduce_ref, row_lse2_ref
+from tests import _inputs
+
+pytestmark = pytest.mark.gpu
+REDUCTIONS = ["sum", "mean", "max"]
+
+
+def check(got: torch.Tensor, want: torch.Tensor, reduction: str, what=""):
+    got = got.detach().float().cpu()
+    want = want.float()
+    assert got.shape == want.shape, (got.shape, want.shape)
+    assert torch.isfinite(got).all(), what
+    if reduction == "max":
+        rel = ((got - want).abs() / want.abs().clamp_min(1e-30)).max().item()
+        assert rel <= 2e-3, f"{what} max: relative error {rel:.3e}"
+    else:
+        torch.testing.assert_close(got, want, rtol=2e-3, atol=1e-5, msg=lambda m: f"{what} {reduction}: {m}")
+
+
+def run_all(q, k, causal, scale=None, what="", reductions=REDUCTIONS, chunk_rows=4096):
+    qd, kd = q.cuda(), k.cuda()
+    for red in reductions:
+        got = fca.flash_colreduce(qd, kd, red, is_causal=causal, scale=scale, out_dtype=torch.float32)
+        want = colreduce_ref(q, k, red, causal, scale=scale, chunk_rows=chunk_rows)
+        check(got, want, red, f"{what} causal={causal}")
+
+
+# --- the reference's own grid (tests/test_correctness.py:8-13), all fp16 ----------------------
+@pytest.mark.parametrize("is_causal", [False, True])
+@pytest.mark.parametrize("d", [16, 32, 64, 48, 72])
+@pytest.mark.parametrize("m,n", [(128, 128), (131, 131), (128, 1024), (131, 1027)])
+@pytest.mark.parametrize("h", [8, 13])
+@pytest.mark.parametrize("b", [1, 4, 7])
+def test_reference_grid(b, h, m, n, d, is_causal):
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=0)
+    run_all(q, k, is_causal, what=f"b{b} h{h} m{m} n{n} d{d}")
+
+
+@pytest.mark.parametrize("is_causal", [False, True])
+@pytest.mark.parametrize("reduction", REDUCTIONS)
+@pytest.mark.parametrize("m,n,d", [(128, 128, 64), (131, 1027, 72), (128, 1024, 48)])
+def test_reference_tolerance_on_native_dtype(m, n, d, reduction, is_causal):
+    """The reference's assertion as written (tests/test_correctness.py:29-32): fp16 result against
+    the materialising implementation run in fp16 on the same device, atol = rtol = 1e-3."""
+    q, k = _inputs.randn_pair(4, 8, m, n, d, seed=0)
+    q, k = q.cuda(), k.cuda()
+    output = fca.flash_colreduce(q, k, reduction=reduction, is_causal=is_causal)
+    target = fca.naive_colreduce(q, k, reduction=reduction, is_causal=is_causal)
+    assert output.dtype == torch.float16 and output.shape == (4, 8, n)
+    torch.testing.assert_close(output, target, atol=1e-3, rtol=1e-3)
+
+
+# --- BASELINE.json configurations ---------------------------------------------------------------
+def test_config1_rounded_to_fp16():
+    """Config 1 is the fp32 CPU case; the device path takes 16-bit inputs, so the kernel is fed
+    the fp16 rounding of the same tensors and compared with the oracle on those."""
+    q, k = _inputs.config1()
+    run_all(q.half(), k.half(), False, what="config1")
+
+
+def test_config2():
+    q, k = _inputs.config2()
+    run_all(q, k, False, what="config2")
+
+
+def test_config3():
+    q, k = _inputs.config3()
+    run_all(q, k, True, what="config3")
+
+
+def _full_size(q, k, reductions, oracle_heads, what):
+    """Full-size run: every head on the GPU, the oracle on a few heads, and properties that
+    hold at any size on all heads (rows of a softmax add to one; 0 < max <= 1; mean <= max)."""
+    m, n = q.shape[2], k.shape[2]
+    qd, kd = q.cuda(), k.cuda()
+    outs = {r: fca.flash_colreduce(qd, kd, r, is_causal=True, out_dtype=torch.float32) for r in reductions}
+    for r, got in outs.items():
+        want = colreduce_ref(q[:, oracle_heads], k[:, oracle_heads], r, True)
+        check(got[:, oracle_heads], want, r, f"{what} heads {oracle_heads}")
+    if "sum" in outs or "mean" in outs:
+        if "sum" in outs:
+            s = outs["sum"].double()
+        else:
+            cnt = torch.arange(n, 0, -1, device="cuda", dtype=torch.float64) if m == n else None
+            s = outs["mean"].double() * cnt
+        total = s.sum(-1).cpu()
+        torch.testing.assert_close(total, torch.full_like(total, float(m)), rtol=1e-4, atol=0)
+    if "max" in outs:
+        mx = outs["max"]
+        assert (mx > 0).all() and (mx <= 1 + 1e-6).all()
+        # causal, M == N: only the last query sees the last key, so max == sum == mean there
+        if "mean" in outs:
+            assert (outs["mean"] <= mx * (1 + 1e-5)).all()
+            torch.testing.assert_close(outs["mean"][..., -1], mx[..., -1], rtol=1e-5, atol=0)
+
+
+def test_config4_full_size():
+    q, k = _inputs.config4()
+    _full_size(q, k, ["sum"], [0, 31], "config4")
+
+
+def test_config5_full_size():
+    q, k = _inputs.config5()
+    _full_size(q, k, ["mean", "max"], [17], "config5")
+
+
+def test_headline_shape_fp16():
+    q, k = _inputs.headline()
+    _full_size(q, k, ["sum"], [5], "headline")
+
+
+# --- beyond the reference's grid ----------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n,d", [
+    (1, 1, 8), (1, 77, 16), (77, 1, 24), (2, 300, 128), (300, 2, 128), (257, 255, 128),
+    (64, 64, 128), (513, 513, 96), (1000, 40, 40), (40, 1000, 20), (333, 777, 104), (700, 300, 56),
+])
+def test_ragged_shapes(m, n, d, causal, dtype):
+    """M > N (offset clamps to 0), single rows/columns, D that needs zero padding, both dtypes."""
+    q, k = _inputs.randn_pair(2, 3, m, n, d, seed=m * 7 + n, dtype=dtype)
+    run_all(q, k, causal, what=f"m{m} n{n} d{d} {dtype}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_explicit_and_negative_scale(causal):
+    q, k = _inputs.randn_pair(1, 4, 200, 333, 64, seed=21)
+    for scale in (0.05, 1.0 / 3.0, -0.125, 0.0):
+        run_all(q, k, causal, scale=scale, what=f"scale={scale}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_strided_inputs(causal):
+    """[B,M,H,D] storage viewed as [B,H,M,D], a slice with a storage offset, and a layout that
+    forces a copy (d stride 2)."""
+    g = torch.Generator().manual_seed(5)
+    b, h, m, n, d = 2, 5, 150, 290, 64
+    q_store = torch.randn(b, m, h, d, generator=g).half()
+    k_store = torch.randn(b, n + 16, h, 2 * d, generator=g).half()
+    q = q_store.permute(0, 2, 1, 3)
+    k = k_store.permute(0, 2, 1, 3)[:, :, 8:8 + n, d:]
+    assert not q.is_contiguous() and not k.is_contiguous()
+    run_all(q, k, causal, what="permuted+sliced")
+    k2 = torch.randn(b, h, n, 2 * d, generator=g).half()[..., ::2]
+    assert k2.stride(3) == 2
+    run_all(q, k2, causal, what="d-stride 2")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_score_jumps_renormalise(causal):
+    """Scores that jump by far more than 64 binades in the middle of the sweep, and rows whose
+    scores are all hugely negative: exercises the renormalisation of the running row sum."""
+    b, h, m, n, d = 1, 2, 96, 640, 64
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=9)
+    q = q.float()
+    k = k.float()
+    k[:, 0, 300] = 40.0 * q[:, 0, 50]          # one enormous aligned key, late
+    k[:, 0, 301] = -40.0 * q[:, 0, 50]         # and an enormously negative one
+    k[:, 1, :, :] = -3.0 * q[:, 1, :1, :] + 0.1 * k[:, 1]   # all scores of row 0 around -190
+    k[:, 1, 500:] *= 0.0
+    run_all(q.half(), k.half(), causal, what="jumps")
+    run_all(q.half(), k.half(), causal, scale=1.0, what="jumps scale 1")
+
+
+def test_heavy_hitter_columns_small():
+    q, k = _inputs.config4(heads=2, n=1024)
+    run_all(q, k, True, what="config4-small")
+    q, k = _inputs.config5(heads=2, n=1536)
+    run_all(q, k, True, what="config5-small")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_row_lse2(causal):
+    q, k = _inputs.randn_pair(2, 3, 300, 520, 80, seed=13)
+    got = fca.row_lse2(q.cuda(), k.cuda(), is_causal=causal).double().cpu()
+    want = row_lse2_ref(q, k, causal)
+    assert got.shape == (2, 3, 300)
+    torch.testing.assert_close(got, want, rtol=0, atol=2e-5 * 12)
+
+
+def test_key_shift_invariance_bf16_inputs():
+    """Adding one vector to every key of a head only shifts each row's scores (config 5's
+    perturbation); exact in real arithmetic, so checked in fp16 where the shift is representable."""
+    q, k = _inputs.randn_pair(1, 2, 256, 384, 64, seed=31)
+    k = (k.float() * 4).round() / 4
+    shift = torch.tensor([0.5, -0.25] * 32).view(1, 1, 1, 64)
+    a = fca.flash_colreduce(q.cuda(), k.half().cuda(), "sum", True, out_dtype=torch.float32)
+    b = fca.flash_colreduce(q.cuda(), (k + shift).half().cuda(), "sum", True, out_dtype=torch.float32)
+    torch.testing.assert_close(a, b, rtol=2e-3, atol=1e-5)
+
+
+def test_deterministic_and_stream_safe():
+    """No atomics: results are bitwise repeatable, also on a side stream."""
+    q, k = _inputs.randn_pair(2, 4, 700, 900, 128, seed=17)
+    q, k = q.cuda(), k.cuda()
+    ref = {r: fca.flash_colreduce(q, k, r, True, out_dtype=torch.float32) for r in REDUCTIONS}
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        again = {r: fca.flash_colreduce(q, k, r, True, out_dtype=torch.float32) for r in REDUCTIONS}
+    s.synchronize()
+    for r in REDUCTIONS:
+        assert torch.equal(ref[r], again[r]), r
+
+
+def test_output_dtype_and_mean_epilogue():
+    q, k = _inputs.randn_pair(1, 2, 64, 200, 32, seed=3, dtype=torch.bfloat16)
+    q, k = q.cuda(), k.cuda()
+    out = fca.flash_colreduce(q, k, "mean", True)
+    assert out.dtype == torch.bfloat16 and out.shape == (1, 2, 200)
+    s = fca.flash_colreduce(q, k, "sum", True)
+    div = torch.cat([torch.full((136,), 64.0), torch.arange(64, 0, -1).float()]).cuda()
+    torch.testing.assert_close(out, (s / div.to(torch.bfloat16)), rtol=0, atol=0)
+
+
+def test_python_errors_on_device():
+    q = torch.zeros(1, 2, 4, 8, dtype=torch.float16, device="cuda")
+    k = torch.zeros(1, 2, 6, 8, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError, match="Invalid reduction: median"):
+        fca.flash_colreduce(q, k, "median")
+    with pytest.raises(ValueError, match="same batch size, number of heads, and head dimension"):
+        fca.flash_colreduce(q, k[:, :1], "sum")
+    with pytest.raises(ValueError, match="float16 or bfloat16"):
+        fca.flash_colreduce(q.float(), k.float(), "sum")
+    # zero queries see no key: every column is 1/N
+    out = fca.flash_colreduce(q, k, "max", out_dtype=torch.float32)
+    torch.testing.assert_close(out, torch.full((1, 2, 6), 1 / 6, device="cuda"))
+    assert fca.flash_colreduce(q[:, :, :0], k, "sum").shape == (1, 2, 6)
+    assert fca.flash_colreduce(q, k[:, :, :0], "sum").shape == (1, 2, 0)
