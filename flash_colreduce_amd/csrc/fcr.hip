@@ -174,13 +174,14 @@ __device__ __forceinline__ void lse_update(const f32x16& acc, float scale2, floa
   float tmax = t[0];
 #pragma unroll
   for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, t[r]);
-  float delta;
-  if (l == 0.f) delta = (tmax > kNegInf) ? tmax : 0.f;
-  else delta = fmaxf(tmax, 0.f);
+  // Nothing seen yet: the tile maximum becomes the reference (it may be far below zero, so the
+  // empty sum must not be scaled: 0 * 2^(+big) is not a number).  Otherwise only ever move up.
+  const bool empty = (l == 0.f);
+  const float delta = empty ? ((tmax > kNegInf) ? tmax : 0.f) : fmaxf(tmax, 0.f);
   float s = 0.f;
 #pragma unroll
   for (int r = 0; r < 16; ++r) s += fast_exp2(t[r] - delta);
-  l = l * fast_exp2(-delta) + s;
+  l = empty ? s : l * fast_exp2(-delta) + s;
   mref += delta;
 }
 
