@@ -34,7 +34,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
 constexpr int kWaveRows = 64;                 // resident rows per wave: two 32-row MFMA blocks
-constexpr int kTileRows = kWaves * kWaveRows; // resident rows per workgroup
+constexpr int kTileRows = kWaves * kWaveRows; // resident rows per workgroup (eight blocks)
 constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row blocks)
 constexpr float kNegInf = -__builtin_inff();
 constexpr float kPosInf = __builtin_inff();
@@ -51,7 +51,8 @@ struct Params {
   int c;             // max(N - M, 0): the causal right-alignment offset
   float scale2;      // scale * log2(e)
   int tiles;         // resident tiles per (b,h)
-  int total;         // tiles * B * H
+  int bh_count;      // B * H
+  int total;         // tiles * B * H workgroups
 };
 
 template <int DT>
@@ -71,70 +72,107 @@ __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_lo
 // Key offset inside a 32-row block of accumulator register r, before the 4*(lane/32) term.
 __device__ __forceinline__ constexpr int reg_row(int r) { return 8 * (r >> 2) + (r & 3); }
 
-// Workgroups are dealt to the 8 XCDs round-robin by blockIdx.  Give each XCD a contiguous run
-// of (b,h) so that the streamed operand of a head stays in one XCD's L2, and inside a head hand
-// out the tiles with the longest sweep first.
-__device__ __forceinline__ bool map_block(const Params& p, bool reverse, int& bh, int& tile) {
-  const int per = (p.total + 7) >> 3;
-  const int v = (int)(blockIdx.x & 7) * per + (int)(blockIdx.x >> 3);
-  if (v >= p.total) return false;
-  bh = v / p.tiles;
-  const int t = v - bh * p.tiles;
-  tile = reverse ? p.tiles - 1 - t : t;
-  return true;
+// Work order.  Workgroup v takes (b,h) = v % BH and the tile of rank v / BH, tiles ranked by the
+// length of their sweep, longest first: with more workgroups than the chip holds at once, the
+// short ones fill in behind the long ones and the causal triangle finishes level.  Workgroups are
+// dealt to the 8 XCDs round-robin by v, so when BH is a multiple of 8 every (b,h) stays on XCD
+// (b,h) % 8 and its streamed operand is shared through that XCD's L2.
+__device__ __forceinline__ void map_block(const Params& p, bool longest_is_last_tile, int& bh, int& tile) {
+  const int v = (int)blockIdx.x;
+  const int rank = v / p.bh_count;
+  bh = v - rank * p.bh_count;
+  tile = longest_is_last_tile ? p.tiles - 1 - rank : rank;
 }
 
-// The operand a wave keeps for the whole sweep: rows [row0, row0+64), as MFMA fragments.
-// Lane l holds, for k-step ks, the 8 elements [16*ks + 8*(l/32), +8) of row (l & 31) of a block.
+// A workgroup's 256 resident rows are eight 32-row blocks; wave w keeps blocks w and 7-w.  On a
+// causal diagonal block b has b+1 (rows) or 8-b (columns) visible sub-tiles out of 8, so every wave
+// gets 9 of the 36 and the four waves reach each barrier together.
+__device__ __forceinline__ void wave_blocks(int tile, int wave, int (&rows)[2]) {
+  rows[0] = tile * kTileRows + 32 * wave;
+  rows[1] = tile * kTileRows + 32 * (7 - wave);
+}
+
+// Raw buffer view of rows [row0, nrows) of a row-major operand.  Loads through it return zero
+// past the last row instead of faulting, so ragged tails need neither branches nor clamps.
+// Offsets inside the view are 32 bit; the host checks that 64 rows fit.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_view(const char* base, int64_t row_bytes, int row0,
+                                                            int nrows) {
+  int64_t bytes = (int64_t)(nrows - row0) * row_bytes;
+  bytes = bytes < 0 ? 0 : (bytes > 0xffffffffll ? 0xffffffffll : bytes);
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base) + (int64_t)row0 * row_bytes, 0,
+                                           (int)(uint32_t)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ u32x4 view_load16(__amdgpu_buffer_rsrc_t v, uint32_t byte_off) {
+  return __builtin_amdgcn_raw_buffer_load_b128(v, (int)byte_off, 0, 0);
+}
+
+// The operand a wave keeps for the whole sweep: two blocks of 32 rows starting at rows[0] and
+// rows[1], as MFMA fragments.  Lane l holds, for k-step ks, the 8 elements
+// [16*ks + 8*(l/32), +8) of row (l & 31) of a block.
 template <int KS>
 __device__ __forceinline__ void load_resident(u32x4 (&f)[2][KS], const char* base, int64_t row_bytes,
-                                              int row0, int nrows, int dgran, int lane) {
+                                              const int (&rows)[2], int nrows, int dgran, int lane) {
+  const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
   for (int blk = 0; blk < 2; ++blk) {
-    const int row = row0 + blk * 32 + (lane & 31);
-    const char* src = base + (int64_t)row * row_bytes;
+    const __amdgpu_buffer_rsrc_t view = rows_view(base, row_bytes, rows[blk], nrows);
+    const uint32_t roff = (uint32_t)(lane & 31) * (uint32_t)row_bytes;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int g = ks * 2 + (lane >> 5);
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (row < nrows && g < dgran) v = *reinterpret_cast<const u32x4*>(src + g * 16);
-      f[blk][ks] = v;
+      const u32x4 v = view_load16(view, roff + (uint32_t)min(g, dgran - 1) * 16u);
+      f[blk][ks] = (g < dgran) ? v : zero;  // zero padding of D up to the k-step
     }
   }
 }
 
 // Global -> registers -> LDS staging of kChunk rows of the streamed operand.
 // LDS rows are padded by 16 bytes so that the 16-byte fragment reads of 16 consecutive rows
-// fall into distinct banks.
+// fall into distinct banks.  A thread moves the same granules (row r, 16-byte column cg) of
+// every chunk, so its source offset inside a chunk and its LDS offset are computed once.
+// Granule columns at or past D/8 (the zero padding up to the MFMA k-step) are never written
+// (their threads store to a dummy slot): the buffers are cleared once and those columns stay zero.
+// Rows past the end of the operand come back as zeros from the buffer view.
 template <int KS>
 struct Stager {
   static constexpr int kGran = 2 * KS;             // 16-byte granules per (zero padded) row
   static constexpr int kRowBytes = KS * 32 + 16;   // LDS row pitch
   static constexpr int kTotal = kChunk * kGran;
   static constexpr int kPer = (kTotal + kThreads - 1) / kThreads;
-  static constexpr int kBytes = kChunk * kRowBytes;
+  static constexpr int kDummy = kChunk * kRowBytes;  // 16 bytes nobody reads
+  static constexpr int kBytes = kChunk * kRowBytes + 16;
   u32x4 regs[kPer];
+  uint32_t goff[kPer];   // source byte offset inside a chunk
+  uint32_t loff[kPer];   // LDS byte offset inside a stage buffer (kDummy for padding granules)
 
-  __device__ __forceinline__ void load(const char* base, int64_t row_bytes, int row0, int nrows,
-                                       int dgran, int tid) {
+  __device__ __forceinline__ void init(int64_t row_bytes, int dgran, int tid) {
 #pragma unroll
     for (int i = 0; i < kPer; ++i) {
       const int g = tid + i * kThreads;
-      const int r = g / kGran, cg = g - r * kGran;
-      const int row = row0 + r;
-      u32x4 v = {0u, 0u, 0u, 0u};
-      if (g < kTotal && row < nrows && cg < dgran)
-        v = *reinterpret_cast<const u32x4*>(base + (int64_t)row * row_bytes + cg * 16);
-      regs[i] = v;
+      const int r = min(g / kGran, kChunk - 1), cg = g % kGran;
+      const bool live = (g < kTotal) && (cg < dgran);
+      goff[i] = (uint32_t)r * (uint32_t)row_bytes + (uint32_t)min(cg, dgran - 1) * 16u;
+      loff[i] = live ? (uint32_t)(r * kRowBytes + cg * 16) : (uint32_t)kDummy;
     }
   }
-  __device__ __forceinline__ void store(char* lds, int tid) const {
-#pragma unroll
-    for (int i = 0; i < kPer; ++i) {
-      const int g = tid + i * kThreads;
-      const int r = g / kGran, cg = g - r * kGran;
-      if (g < kTotal) *reinterpret_cast<u32x4*>(lds + r * kRowBytes + cg * 16) = regs[i];
+  // Clears `bytes` of LDS (a multiple of 16) when some granule columns are padding.
+  static __device__ __forceinline__ void clear(char* lds, int bytes, int dgran, int tid) {
+    if (dgran < kGran) {
+      const u32x4 zero = {0u, 0u, 0u, 0u};
+      for (int o = tid * 16; o < bytes; o += kThreads * 16) *reinterpret_cast<u32x4*>(lds + o) = zero;
+      __syncthreads();
     }
+  }
+  // Rows [row0, row0 + kChunk) of an operand of nrows rows starting at base.  No branches.
+  __device__ __forceinline__ void load(const char* base, int64_t row_bytes, int row0, int nrows) {
+    const __amdgpu_buffer_rsrc_t view = rows_view(base, row_bytes, row0, nrows);
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) regs[i] = view_load16(view, goff[i]);
+  }
+  __device__ __forceinline__ void store(char* lds) const {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) *reinterpret_cast<u32x4*>(lds + loff[i]) = regs[i];
   }
   // Fragment of block `sub` (32 rows) for k-step ks.
   static __device__ __forceinline__ u32x4 frag(const char* lds, int sub, int ks, int lane) {
@@ -143,33 +181,118 @@ struct Stager {
   }
 };
 
+// One sub-step of a sweep: 32 streamed rows (fragments f) against the wave's 64 resident rows, as
+// two independent accumulator chains.  S^T = K * Q^T, so keys are the A operand.  When REFILL, each
+// fragment register is reloaded for the sub-step after this one as soon as its MFMAs are issued, a
+// whole sub-step ahead of its use.
+template <int DT, int KS, bool RESIDENT_IS_KEYS, bool REFILL>
+__device__ __forceinline__ void mma_pair(f32x16& n0, f32x16& n1, u32x4 (&f)[KS], const u32x4 (&res)[2][KS],
+                                         const char* next_lds, int next_sub, int lane) {
+  using St = Stager<KS>;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { n0[r] = 0.f; n1[r] = 0.f; }
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) {
+    if (RESIDENT_IS_KEYS) {
+      n0 = mma<DT>(res[0][ks], f[ks], n0);
+      n1 = mma<DT>(res[1][ks], f[ks], n1);
+    } else {
+      n0 = mma<DT>(f[ks], res[0][ks], n0);
+      n1 = mma<DT>(f[ks], res[1][ks], n1);
+    }
+    if (REFILL) f[ks] = St::frag(next_lds, next_sub, ks, lane);
+  }
+}
+
+// Branch-free sweep over chunks [ta, tb) of the streamed operand, none of which needs a mask.
+// Chunk t lives in stage buffer t & 1.  On entry chunk ta has been stored to its buffer (not yet
+// published by a barrier) and the staging registers hold chunk ta+1; on exit the same holds for tb,
+// so the general loops can run before or after.
+//
+// Steady state, per chunk t (two sub-steps s0, s1), one barrier:
+//     barrier            chunk t+1 published; nobody reads chunk t from LDS any more
+//     MFMA(s1 of t)   || VALU of s0 of t   || fragments <- s0 of t+1   || stage t+2: regs -> LDS,
+//     MFMA(s0 of t+1) || VALU of s1 of t   || fragments <- s1 of t+1   || regs <- chunk t+3
+// Every LDS read is issued a sub-step before its use, every global load a chunk before its store,
+// every LDS store half a chunk before the barrier that publishes it.
+// aux_of(lds, sub) reads what the consumer needs per sub-step besides the scores (the column
+// kernel: -lse of the lane's query); it travels with the fragments so that it too is read before
+// the barrier that lets other waves overwrite the buffer.
+template <int DT, int KS, bool RESIDENT_IS_KEYS, class StoreF, class LoadF, class AuxF, class ConsumeF>
+__device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[2][KS], char* smem,
+                                                int stage_bytes, int lane, StoreF&& stage_store,
+                                                LoadF&& stage_load, AuxF&& aux_of, ConsumeF&& consume) {
+  using St = Stager<KS>;
+  if (ta >= tb) return;
+  u32x4 f[KS];
+  f32x16 p0, p1, n0, n1;
+  float af, ap, an;
+  __syncthreads();
+  stage_store(smem + ((ta + 1) & 1) * stage_bytes);
+  stage_load(ta + 2);
+  {
+    const char* lds = smem + (ta & 1) * stage_bytes;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) f[ks] = St::frag(lds, 0, ks, lane);
+    ap = aux_of(lds, 0);
+    mma_pair<DT, KS, RESIDENT_IS_KEYS, true>(p0, p1, f, res, lds, 1, lane);
+    af = aux_of(lds, 1);
+  }
+  for (int t = ta; t + 1 < tb; ++t) {
+    const char* nxt = smem + ((t + 1) & 1) * stage_bytes;
+    __syncthreads();
+    an = af;
+    mma_pair<DT, KS, RESIDENT_IS_KEYS, true>(n0, n1, f, res, nxt, 0, lane);
+    af = aux_of(nxt, 0);
+    consume(p0, p1, ap);
+    p0 = n0; p1 = n1; ap = an;
+    stage_store(smem + (t & 1) * stage_bytes);
+    stage_load(t + 3);
+    an = af;
+    mma_pair<DT, KS, RESIDENT_IS_KEYS, true>(n0, n1, f, res, nxt, 1, lane);
+    af = aux_of(nxt, 1);
+    consume(p0, p1, ap);
+    p0 = n0; p1 = n1; ap = an;
+  }
+  mma_pair<DT, KS, RESIDENT_IS_KEYS, false>(n0, n1, f, res, nullptr, 0, lane);
+  consume(p0, p1, ap);
+  consume(n0, n1, af);
+}
+
 // ---------------------------------------------------------------------------------------------
 // Row statistics.  Per lane and 32-query block the state is (mref, l) with
 //   sum over the keys seen so far of 2^(s) = l * 2^mref.
-// mref is a reference exponent, not the running maximum: the common path adds 2^(s - mref)
-// without looking for a maximum.  The sum is renormalised only when it leaves [1, 2^64) -- the
-// first visible keys of a row, or a jump of the scores by more than 64 binades -- and then
-// exactly as the classic online softmax would (new reference = old + max(tile max, 0)).
-// Invariant after the first visible key: 1 <= l < 2^64, hence mref <= lse < mref + 64, so terms
-// that underflow are below 2^-126 of the total and overflow is caught by the range check.
+// mref is a reference exponent, not the running maximum: the common path (lse_fast) adds
+// 2^(s - mref) without looking for a maximum.  The sum is renormalised (lse_renorm) only when it
+// leaves [1, 2^64) -- the first visible keys of a row, or a jump of the scores by more than 64
+// binades -- and then exactly as the classic online softmax would (new reference = old +
+// max(tile max, 0)).  Invariant after the first visible key: 1 <= l < 2^64, hence
+// mref <= lse < mref + 64, so terms that underflow are below 2^-126 of the total and overflow is
+// caught by the range check.
 template <bool MASK>
-__device__ __forceinline__ void lse_update(const f32x16& acc, float scale2, float& mref, float& l,
-                                           int lim) {
+__device__ __forceinline__ float lse_fast(const f32x16& acc, float scale2, float mref, float l, int lim) {
   const float nm = -mref;
-  float t[16];
   float s0 = 0.f, s1 = 0.f;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     float x = fmaf(acc[r], scale2, nm);
     if (MASK) x = (reg_row(r) <= lim) ? x : kNegInf;
-    t[r] = x;
     if (r & 1) s1 += fast_exp2(x); else s0 += fast_exp2(x);
   }
-  const float ln = l + (s0 + s1);
-  const bool ok = (ln >= 1.0f) && (ln < 1.8446744e19f);
-  if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
-    l = ln;
-    return;
+  return l + (s0 + s1);
+}
+
+__device__ __forceinline__ bool lse_in_range(float l) { return (l >= 1.0f) && (l < 1.8446744e19f); }
+
+template <bool MASK>
+__device__ __forceinline__ void lse_renorm(const f32x16& acc, float scale2, float& mref, float& l, int lim) {
+  const float nm = -mref;
+  float t[16];
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    float x = fmaf(acc[r], scale2, nm);
+    if (MASK) x = (reg_row(r) <= lim) ? x : kNegInf;
+    t[r] = x;
   }
   float tmax = t[0];
 #pragma unroll
@@ -185,6 +308,28 @@ __device__ __forceinline__ void lse_update(const f32x16& acc, float scale2, floa
   mref += delta;
 }
 
+template <bool MASK>
+__device__ __forceinline__ void lse_update(const f32x16& acc, float scale2, float& mref, float& l, int lim) {
+  const float ln = lse_fast<MASK>(acc, scale2, mref, l, lim);
+  if (__builtin_amdgcn_ballot_w64(!lse_in_range(ln)) == 0) l = ln;
+  else lse_renorm<MASK>(acc, scale2, mref, l, lim);
+}
+
+// Both blocks of a fully visible sub-step; one rarely taken branch at the very end so that the
+// arithmetic above it can be scheduled against the MFMAs of the next sub-step.
+__device__ __forceinline__ void lse_update_pair(const f32x16& a0, const f32x16& a1, float scale2,
+                                                float (&mref)[2], float (&l)[2]) {
+  const float ln0 = lse_fast<false>(a0, scale2, mref[0], l[0], 0);
+  const float ln1 = lse_fast<false>(a1, scale2, mref[1], l[1], 0);
+  if (__builtin_amdgcn_ballot_w64(!(lse_in_range(ln0) && lse_in_range(ln1))) == 0) {
+    l[0] = ln0;
+    l[1] = ln1;
+  } else {
+    lse_renorm<false>(a0, scale2, mref[0], l[0], 0);
+    lse_renorm<false>(a1, scale2, mref[1], l[1], 0);
+  }
+}
+
 __device__ __forceinline__ float lse_merge(float a, float b) {
   const float hi = fmaxf(a, b), lo = fminf(a, b);
   if (hi == kNegInf) return kNegInf;
@@ -196,44 +341,58 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   using St = Stager<KS>;
   __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
   int bh, tile;
-  if (!map_block(p, CAUSAL, bh, tile)) return;
+  map_block(p, CAUSAL, bh, tile);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int b = bh / p.H, h = bh - b * p.H;
   const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
   const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
 
-  const int q0 = tile * kTileRows + wave * kWaveRows;  // first query of this wave
+  int q0[2];  // first query of each of this wave's blocks
+  wave_blocks(tile, wave, q0);
   u32x4 qf[2][KS];
   load_resident<KS>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
 
-  // keys this workgroup / this wave has to look at
-  const int kend_wg = CAUSAL ? min(p.N, tile * kTileRows + kTileRows + p.c) : p.N;
-  const int nchunks = (kend_wg + kChunk - 1) / kChunk;
+  // Keys [0, kend) matter to this workgroup.  Chunks [0, t_int) are seen in full by every one of
+  // its queries and lie inside [0, N): they take the branch-free pipelined sweep.  The rest (the
+  // causal diagonal, the ragged tail) take the general loop.
+  const int kend = CAUSAL ? min(p.N, tile * kTileRows + kTileRows + p.c) : p.N;
+  const int nchunks = (kend + kChunk - 1) / kChunk;
+  const int t_int = CAUSAL ? min((tile * kTileRows + p.c + 1) / kChunk, p.N / kChunk) : p.N / kChunk;
 
   float mref[2] = {0.f, 0.f}, l[2] = {0.f, 0.f};
-  // last key a lane's query may see, per block
-  int last[2];
+  int last[2];  // last key a lane's query may see, minus the lane's row offset in a block
 #pragma unroll
   for (int blk = 0; blk < 2; ++blk) {
-    const int i = q0 + blk * 32 + (lane & 31);
+    const int i = q0[blk] + (lane & 31);
     last[blk] = (CAUSAL ? min(p.N - 1, i + p.c) : p.N - 1) - 4 * (lane >> 5);
   }
 
   St st;
-  st.load(kb, p.k_sr, 0, p.N, p.dgran, tid);
-  int buf = 0;
-  for (int t = 0; t < nchunks; ++t) {
-    char* lds = smem + buf * St::kBytes;
-    st.store(lds, tid);
-    __syncthreads();
-    if (t + 1 < nchunks) st.load(kb, p.k_sr, (t + 1) * kChunk, p.N, p.dgran, tid);
+  st.init(p.k_sr, p.dgran, tid);
+  St::clear(smem, 2 * St::kBytes, p.dgran, tid);
+  auto stage_store = [&](char* lds) { st.store(lds); };
+  auto stage_load = [&](int t) { st.load(kb, p.k_sr, t * kChunk, p.N); };
+  stage_load(0);
+  stage_store(smem);
+  stage_load(1);
+
+  pipelined_sweep<DT, KS, false>(
+      0, t_int, qf, smem, St::kBytes, lane, stage_store, stage_load,
+      [](const char*, int) { return 0.f; },
+      [&](const f32x16& a0, const f32x16& a1, float) { lse_update_pair(a0, a1, p.scale2, mref, l); });
+
+  for (int t = t_int; t < nchunks; ++t) {
+    __syncthreads();  // chunk t published, the other buffer is free
+    stage_store(smem + ((t + 1) & 1) * St::kBytes);
+    stage_load(t + 2);
+    const char* lds = smem + (t & 1) * St::kBytes;
 #pragma unroll
     for (int sub = 0; sub < kChunk / 32; ++sub) {
       const int key0 = t * kChunk + sub * 32;
       if (key0 >= p.N) continue;
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk) {
-        const int qblk = q0 + blk * 32;
+        const int qblk = q0[blk];
         if (CAUSAL && key0 > qblk + 31 + p.c) continue;  // block cannot see this sub-tile
         f32x16 acc = {0};
 #pragma unroll
@@ -243,7 +402,6 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
         else lse_update<false>(acc, p.scale2, mref[blk], l[blk], 0);
       }
     }
-    buf ^= 1;
   }
 
 #pragma unroll
@@ -251,7 +409,7 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
     float v = (l[blk] > 0.f) ? mref[blk] + fast_log2(l[blk]) : kNegInf;
     const float o = __shfl_xor(v, 32);
     v = lse_merge(v, o);
-    const int i = q0 + blk * 32 + lane;
+    const int i = q0[blk] + lane;
     if (lane < 32 && i < p.M) p.lse[(int64_t)bh * p.M + i] = v;
   }
 }
@@ -277,14 +435,15 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
   constexpr int kSmem = (2 * kStage > kRed) ? 2 * kStage : kRed;
   __shared__ __attribute__((aligned(16))) char smem[kSmem];
   int bh, tile;
-  if (!map_block(p, false, bh, tile)) return;
+  map_block(p, false, bh, tile);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int b = bh / p.H, h = bh - b * p.H;
   const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
   const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
   const float* lse = p.lse + (int64_t)bh * p.M;
 
-  const int k0 = tile * kTileRows + wave * kWaveRows;  // first key of this wave
+  int k0[2];  // first key of each of this wave's blocks
+  wave_blocks(tile, wave, k0);
   u32x4 kf[2][KS];
   load_resident<KS>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
 
@@ -294,35 +453,43 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
 #pragma unroll
     for (int r = 0; r < 16; ++r) col[blk][r] = ISMAX ? kNegInf : 0.f;
 
-  // first query chunk that can see any key of this tile
-  const int t0 = CAUSAL ? max(0, tile * kTileRows - p.c) / kChunk : 0;
+  // Query chunks [t0, nchunks) can see keys of this tile.  From chunk t_int on every query sees
+  // all of them: those chunks take the branch-free pipelined sweep (rows past M carry lse = +inf
+  // and add 2^-inf = 0, keys past N are computed and never stored, so neither needs a mask).
   const int nchunks = (p.M + kChunk - 1) / kChunk;
+  const int t0 = CAUSAL ? max(0, tile * kTileRows - p.c) / kChunk : 0;
+  const int t_int = CAUSAL ? min(nchunks, max(t0, (tile * kTileRows + kTileRows - 1 - p.c + kChunk - 1) / kChunk)) : 0;
   // lim = i + c - key0(blk) - 4*(lane/32), with i the lane's query in the current sub-tile
   const int lim_lane = (lane & 31) + p.c - 4 * (lane >> 5);
 
+  // A stage is kChunk query rows plus their lse.  The lse value loaded for chunk t is first
+  // touched when the stage is stored, a chunk after its load was issued.
   St st;
-  float lse_reg = kPosInf;
-  auto load_lse = [&](int row0) {
-    if (tid < kChunk) {
-      const int i = row0 + tid;
-      lse_reg = (i < p.M) ? lse[i] : kPosInf;  // +inf: rows past M contribute 2^-inf = 0
-    }
+  float lse_reg;
+  bool lse_live;
+  st.init(p.q_sr, p.dgran, tid);
+  St::clear(smem, 2 * kStage, p.dgran, tid);
+  auto stage_load = [&](int t) {
+    st.load(qb, p.q_sr, t * kChunk, p.M);
+    const int i = t * kChunk + (tid & (kChunk - 1));  // threads 64.. duplicate threads 0..63
+    lse_reg = lse[min(i, p.M - 1)];
+    lse_live = (i < p.M);
   };
-  if (t0 < nchunks) {
-    st.load(qb, p.q_sr, t0 * kChunk, p.M, p.dgran, tid);
-    load_lse(t0 * kChunk);
-  }
-  int buf = 0;
-  for (int t = t0; t < nchunks; ++t) {
-    char* lds = smem + buf * kStage;
-    float* lds_lse = reinterpret_cast<float*>(lds + St::kBytes);
-    st.store(lds, tid);
-    if (tid < kChunk) lds_lse[tid] = lse_reg;
-    __syncthreads();
-    if (t + 1 < nchunks) {
-      st.load(qb, p.q_sr, (t + 1) * kChunk, p.M, p.dgran, tid);
-      load_lse((t + 1) * kChunk);
-    }
+  auto stage_store = [&](char* lds) {
+    st.store(lds);
+    // +inf for rows past M: they contribute 2^-inf = 0
+    reinterpret_cast<float*>(lds + St::kBytes)[tid & (kChunk - 1)] = lse_live ? lse_reg : kPosInf;
+  };
+  stage_load(t0);
+  stage_store(smem + (t0 & 1) * kStage);
+  stage_load(t0 + 1);
+
+  for (int t = t0; t < t_int; ++t) {
+    __syncthreads();  // chunk t published, the other buffer is free
+    stage_store(smem + ((t + 1) & 1) * kStage);
+    stage_load(t + 2);
+    const char* lds = smem + (t & 1) * kStage;
+    const float* lds_lse = reinterpret_cast<const float*>(lds + St::kBytes);
 #pragma unroll
     for (int sub = 0; sub < kChunk / 32; ++sub) {
       const int qs = t * kChunk + sub * 32;  // first query of the sub-tile
@@ -330,7 +497,7 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
       const float nlse = -lds_lse[sub * 32 + (lane & 31)];
 #pragma unroll
       for (int blk = 0; blk < 2; ++blk) {
-        const int kblk = k0 + blk * 32;
+        const int kblk = k0[blk];
         if (kblk >= p.N) continue;
         if (CAUSAL && kblk > qs + 31 + p.c) continue;  // no query of the sub-tile sees this block
         f32x16 acc = {0};
@@ -341,8 +508,17 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
         else col_update<false, ISMAX>(acc, p.scale2, nlse, col[blk], 0);
       }
     }
-    buf ^= 1;
   }
+
+  pipelined_sweep<DT, KS, true>(
+      t_int, nchunks, kf, smem, kStage, lane, stage_store, stage_load,
+      [&](const char* lds, int sub) {
+        return -reinterpret_cast<const float*>(lds + St::kBytes)[sub * 32 + (lane & 31)];
+      },
+      [&](const f32x16& a0, const f32x16& a1, float nlse) {
+        col_update<false, ISMAX>(a0, p.scale2, nlse, col[0], 0);
+        col_update<false, ISMAX>(a1, p.scale2, nlse, col[1], 0);
+      });
 
   // Reduce over the 32 query lanes: transpose through LDS, one output key per lane.
   __syncthreads();
@@ -363,7 +539,7 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
       v = ISMAX ? fmaxf(v, x) : v + x;
     }
     if (ISMAX) v = fast_exp2(v);
-    const int key = k0 + lane;
+    const int key = k0[lane >> 5] + w;
     if (key < p.N) p.out[(int64_t)bh * p.N + key] = v;
   }
 }
@@ -382,9 +558,9 @@ int check_strides(const void* ptr, const int64_t s[4], const char* name) {
     return FCR_E_STRIDE;
   }
   if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0 || s[0] % 8 != 0 || s[1] % 8 != 0 || s[2] % 8 != 0 ||
-      s[0] < 0 || s[1] < 0 || s[2] < 0) {
+      s[0] < 0 || s[1] < 0 || s[2] < 0 || s[2] >= (1 << 24)) {
     snprintf(g_err, sizeof(g_err),
-             "%s: base pointer must be 16-byte aligned and batch/head/row strides non-negative multiples of 8 elements",
+             "%s: base pointer must be 16-byte aligned, batch/head/row strides non-negative multiples of 8 elements, row stride < 2^24",
              name);
     return FCR_E_STRIDE;
   }
@@ -415,6 +591,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   p.c = N > M ? N - M : 0;
   p.scale2 = (float)((double)scale * 1.4426950408889634);
   p.tiles = (int)tiles;
+  p.bh_count = (int)bh;
   p.total = (int)(bh * tiles);
   p.lse = nullptr;
   p.out = nullptr;
@@ -430,14 +607,14 @@ int launched(const char* what) {
 
 template <int DT, int KS>
 void launch_lse(const Params& p, bool causal, hipStream_t s) {
-  const dim3 grid(((p.total + 7) / 8) * 8), block(kThreads);
+  const dim3 grid(p.total), block(kThreads);
   if (causal) hipLaunchKernelGGL((row_lse_kernel<DT, KS, true>), grid, block, 0, s, p);
   else hipLaunchKernelGGL((row_lse_kernel<DT, KS, false>), grid, block, 0, s, p);
 }
 
 template <int DT, int KS>
 void launch_col(const Params& p, bool causal, bool ismax, hipStream_t s) {
-  const dim3 grid(((p.total + 7) / 8) * 8), block(kThreads);
+  const dim3 grid(p.total), block(kThreads);
   if (causal) {
     if (ismax) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, true>), grid, block, 0, s, p);
     else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, false>), grid, block, 0, s, p);

@@ -50,7 +50,8 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
     if d % 8 != 0:
         return torch.nn.functional.pad(x, (0, 8 - d % 8))  # new contiguous tensor
     ok = (x.stride(3) == 1 and x.data_ptr() % 16 == 0 and
-          all(x.stride(i) % 8 == 0 and x.stride(i) >= 0 for i in (0, 1, 2)))
+          all(x.stride(i) % 8 == 0 and x.stride(i) >= 0 for i in (0, 1, 2)) and
+          x.stride(2) < (1 << 24))
     return x if ok else x.contiguous()
 
 
