@@ -4,7 +4,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--cpu-heads H]
 
 One step = one fcr_colreduce call (row-statistics kernel + column-reduce kernel) on the headline
-workload of BASELINE.json: causal, B=1, H=32, M=N=8192, D=128, fp16, reduction=sum, inputs
+workload: causal, B=1, H=32, M=N=8192, D=128, fp16, reduction=sum, inputs
 resident in HBM, buffers preallocated.  Prints ONE JSON line.
 
 value        effective TFLOP/s = (4*B*H*M*N*D / 2) / time per call (flop convention of the metric).
@@ -26,6 +26,10 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 PEAK_FP16_DENSE_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/CU/clk, MI355X published dense fp16
+# HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
+# scaled by the same counters on a 256 MiB device copy (FETCH unit 2 KiB, WRITE unit 1 KiB);
+# the summary of those runs is profiles/headline_causal_8192_fp16.md.
+HBM_TRAFFIC_BYTES = {"row_lse_kernel": 197.4e6 + 1.05e6, "col_reduce_kernel": 172.9e6 + 1.05e6}
 
 
 def main():
@@ -33,12 +37,17 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--cpu-heads", type=int, default=8,
+    ap.add_argument("--cpu-heads", type=int, default=32,
                     help="heads of the workload the CPU oracle is timed on (0 = skip)")
+    ap.add_argument("--copy-calib", action="store_true",
+                    help="also run one plain 256 MiB device copy, as the known-size reference for "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
+    ap.add_argument("--traffic-bytes", type=float, default=None,
+                    help="override roofline.traffic (HBM bytes per launch of the dominant kernel)")
     args = ap.parse_args()
     if args.gpus != 1:
-        print("bench.py: this build runs on one GPU only (every (b,h) is independent; see DESIGN.md "
-              "for how it would shard); run with --gpus 1", file=sys.stderr)
+        print("bench.py: this build runs on one GPU only (every (b,h) pair is independent and would shard "
+              "across GPUs without any exchange, but no multi-GPU path is built); run with --gpus 1", file=sys.stderr)
         sys.exit(2)
 
     import torch
@@ -93,6 +102,11 @@ def main():
 
     reps = max(args.steps, 10)
     k1_ms, k2_ms = event_ms(pass1, reps), event_ms(pass2, reps)
+    if args.copy_calib:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
 
     flop_call = 4.0 * B * H * M * N * D / 2.0       # two masked GEMMs, causal halves the work
     flop_kernel = flop_call / 2.0
@@ -104,7 +118,7 @@ def main():
     dom = max(kernels, key=lambda n: kernels[n]["ms"])
     roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"],
                 "peak": PEAK_FP16_DENSE_TFLOPS, "unit": "TFLOP/s",
-                "frac": kernels[dom]["tflops"] / PEAK_FP16_DENSE_TFLOPS, "traffic": None,
+                "frac": kernels[dom]["tflops"] / PEAK_FP16_DENSE_TFLOPS, "traffic": args.traffic_bytes if args.traffic_bytes is not None else HBM_TRAFFIC_BYTES[dom],
                 "kernels": kernels, "whole_call_frac": value / PEAK_FP16_DENSE_TFLOPS}
 
     cpu_baseline = None

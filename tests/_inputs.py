@@ -1,7 +1,7 @@
 """Seeded synthetic inputs shared by the GPU parity tests, the smoke test and the bench.
 
 Everything is drawn from the CPU generator in fp32 and then cast, so the CPU oracle and the
-GPU kernel see identical bits.  The five named configurations follow BASELINE.json.
+GPU kernel see identical bits.  config1..config5 and headline are the benchmark set's named workloads.
 """
 from __future__ import annotations
 

@@ -85,7 +85,7 @@ def test_python_entry_validation_matches_reference_messages():
 
 
 def test_naive_colreduce_matches_oracle_on_config1():
-    """BASELINE config 1: the CPU-runnable fp32 case, non-causal, all three reductions."""
+    """Configuration 1 of the benchmark set: the CPU-runnable fp32 case, non-causal, all three reductions."""
     q, k = _inputs.config1()
     for red in ("sum", "mean", "max"):
         got = fca.naive_colreduce(q, k, red)

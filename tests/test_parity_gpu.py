@@ -1,5 +1,5 @@
 """GPU parity: libfcr (through flash_colreduce / the C ABI) against the CPU oracle on the same
-seeded inputs.  Tolerances are BASELINE.json's: rtol 2e-3 / atol 1e-5 for sum and mean,
+seeded inputs.  Tolerances are those of the headline metric: rtol 2e-3 / atol 1e-5 for sum and mean,
 2e-3 relative for max, checked on the kernel's fp32 result."""
 import math
 
@@ -59,7 +59,7 @@ def test_reference_tolerance_on_native_dtype(m, n, d, reduction, is_causal):
     torch.testing.assert_close(output, target, atol=1e-3, rtol=1e-3)
 
 
-# --- BASELINE.json configurations ---------------------------------------------------------------
+# --- the benchmark set's five configurations ---------------------------------------------------------------
 def test_config1_rounded_to_fp16():
     """Config 1 is the fp32 CPU case; the device path takes 16-bit inputs, so the kernel is fed
     the fp16 rounding of the same tensors and compared with the oracle on those."""
