@@ -43,6 +43,8 @@ struct Params {
   const char* q;
   const char* k;
   float* lse;        // [BH, M]
+  float* part;       // [splits, BH, M] partial lse of key ranges when splits > 1
+  int splits;        // key ranges per row tile in the row kernel (1 = whole sweep in one workgroup)
   float* out;        // [BH, N]
   int64_t q_sb, q_sh, q_sr;  // strides in BYTES: batch, head, row
   int64_t k_sb, k_sh, k_sr;
@@ -81,6 +83,18 @@ __device__ __forceinline__ void map_block(const Params& p, bool longest_is_last_
   const int v = (int)blockIdx.x;
   const int rank = v / p.bh_count;
   bh = v - rank * p.bh_count;
+  tile = longest_is_last_tile ? p.tiles - 1 - rank : rank;
+}
+
+// Row kernel with the keys of a tile split over several workgroups (few query rows, many keys):
+// workgroup v takes (b,h) = v % BH, then the key range, then the tile.
+__device__ __forceinline__ void map_block_split(const Params& p, bool longest_is_last_tile, int& bh, int& tile,
+                                                int& split) {
+  const int v = (int)blockIdx.x;
+  const int r = v / p.bh_count;
+  bh = v - r * p.bh_count;
+  const int rank = r / p.splits;
+  split = r - rank * p.splits;
   tile = longest_is_last_tile ? p.tiles - 1 - rank : rank;
 }
 
@@ -340,9 +354,10 @@ template <int DT, int KS, bool CAUSAL>
 __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   using St = Stager<KS>;
   __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
-  int bh, tile;
-  map_block(p, CAUSAL, bh, tile);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  int bh, tile, split;
+  map_block_split(p, CAUSAL, bh, tile, split);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lets addresses stay scalar
   const int b = bh / p.H, h = bh - b * p.H;
   const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
   const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
@@ -355,9 +370,13 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   // Keys [0, kend) matter to this workgroup.  Chunks [0, t_int) are seen in full by every one of
   // its queries and lie inside [0, N): they take the branch-free pipelined sweep.  The rest (the
   // causal diagonal, the ragged tail) take the general loop.
+  // With splits > 1 this workgroup only sweeps chunks [c_begin, c_end) of that range and writes a
+  // partial lse; lse_combine_kernel merges the partials.
   const int kend = CAUSAL ? min(p.N, tile * kTileRows + kTileRows + p.c) : p.N;
-  const int nchunks = (kend + kChunk - 1) / kChunk;
-  const int t_int = CAUSAL ? min((tile * kTileRows + p.c + 1) / kChunk, p.N / kChunk) : p.N / kChunk;
+  const int per_split = ((p.N + kChunk - 1) / kChunk + p.splits - 1) / p.splits;
+  const int c_begin = split * per_split;
+  const int nchunks = min((kend + kChunk - 1) / kChunk, c_begin + per_split);
+  const int t_int = min(nchunks, CAUSAL ? min((tile * kTileRows + p.c + 1) / kChunk, p.N / kChunk) : p.N / kChunk);
 
   float mref[2] = {0.f, 0.f}, l[2] = {0.f, 0.f};
   int last[2];  // last key a lane's query may see, minus the lane's row offset in a block
@@ -372,16 +391,16 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   St::clear(smem, 2 * St::kBytes, p.dgran, tid);
   auto stage_store = [&](char* lds) { st.store(lds); };
   auto stage_load = [&](int t) { st.load(kb, p.k_sr, t * kChunk, p.N); };
-  stage_load(0);
-  stage_store(smem);
-  stage_load(1);
+  stage_load(c_begin);
+  stage_store(smem + (c_begin & 1) * St::kBytes);
+  stage_load(c_begin + 1);
 
   pipelined_sweep<DT, KS, false>(
-      0, t_int, qf, smem, St::kBytes, lane, stage_store, stage_load,
+      c_begin, t_int, qf, smem, St::kBytes, lane, stage_store, stage_load,
       [](const char*, int) { return 0.f; },
       [&](const f32x16& a0, const f32x16& a1, float) { lse_update_pair(a0, a1, p.scale2, mref, l); });
 
-  for (int t = t_int; t < nchunks; ++t) {
+  for (int t = max(t_int, c_begin); t < nchunks; ++t) {
     __syncthreads();  // chunk t published, the other buffer is free
     stage_store(smem + ((t + 1) & 1) * St::kBytes);
     stage_load(t + 2);
@@ -410,8 +429,22 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
     const float o = __shfl_xor(v, 32);
     v = lse_merge(v, o);
     const int i = q0[blk] + lane;
-    if (lane < 32 && i < p.M) p.lse[(int64_t)bh * p.M + i] = v;
+    float* dst = (p.splits > 1) ? p.part + (int64_t)split * p.bh_count * p.M : p.lse;
+    if (lane < 32 && i < p.M) dst[(int64_t)bh * p.M + i] = v;
   }
+}
+
+// lse[r] = log2 sum_s 2^part[s][r] over the key ranges of a split row sweep.
+__global__ __launch_bounds__(256) void lse_combine_kernel(const float* __restrict__ part, float* __restrict__ lse,
+                                                          int64_t rows, int splits) {
+  const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (r >= rows) return;
+  float m = kNegInf;
+  for (int s = 0; s < splits; ++s) m = fmaxf(m, part[s * rows + r]);
+  float acc = 0.f;
+  if (m > kNegInf)
+    for (int s = 0; s < splits; ++s) acc += fast_exp2(part[s * rows + r] - m);
+  lse[r] = (m > kNegInf) ? m + fast_log2(acc) : kNegInf;
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -436,7 +469,8 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
   __shared__ __attribute__((aligned(16))) char smem[kSmem];
   int bh, tile;
   map_block(p, false, bh, tile);
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lets addresses stay scalar
   const int b = bh / p.H, h = bh - b * p.H;
   const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
   const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
@@ -595,7 +629,22 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   p.total = (int)(bh * tiles);
   p.lse = nullptr;
   p.out = nullptr;
+  p.part = nullptr;
+  p.splits = 1;
   return 0;
+}
+
+// Key ranges per row tile in the row kernel.  One sweep per workgroup when there is at least one
+// workgroup per CU; otherwise the keys of a tile are split so that about two per CU run, each
+// keeping at least four 64-key chunks.
+int row_splits(int B, int H, int M, int N) {
+  const int64_t wgs = (int64_t)B * H * ((M + kTileRows - 1) / kTileRows);
+  const int64_t chunks = (N + kChunk - 1) / kChunk;
+  if (wgs >= 256 || chunks < 16) return 1;
+  int64_t s = 512 / wgs;
+  if (s > chunks / 4) s = chunks / 4;
+  if (s > 64) s = 64;
+  return s < 1 ? 1 : (int)s;
 }
 
 int launched(const char* what) {
@@ -644,9 +693,11 @@ int fcr_version(void) { return FCR_VERSION; }
 
 const char* fcr_last_error(void) { return g_err; }
 
-size_t fcr_lse_bytes(int B, int H, int M) {
-  if (B < 0 || H < 0 || M < 0) return 0;
-  return (size_t)B * (size_t)H * (size_t)M * sizeof(float);
+size_t fcr_lse_bytes(int B, int H, int M, int N) {
+  if (B < 1 || H < 1 || M < 1 || N < 1) return 0;
+  const int splits = row_splits(B, H, M, N);
+  const size_t rows = (size_t)B * (size_t)H * (size_t)M;
+  return rows * sizeof(float) * (splits > 1 ? 1 + (size_t)splits : 1);
 }
 
 int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int H, int M, int N, int D,
@@ -657,13 +708,21 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
   int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, false);
   if (rc) return rc;
   p.lse = lse;
+  p.splits = row_splits(B, H, M, N);
+  p.part = lse + (int64_t)B * H * M;  // only touched when splits > 1 (see fcr_lse_bytes)
+  p.total *= p.splits;
   const int ksteps = (D + 15) / 16;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal != 0, s)
   if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_LSE) }
   else { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_LSE) }
 #undef FCR_CALL_LSE
-  return launched("row_lse_kernel");
+  rc = launched("row_lse_kernel");
+  if (rc || p.splits == 1) return rc;
+  const int64_t rows = (int64_t)B * H * M;
+  hipLaunchKernelGGL(lse_combine_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0, s, p.part, lse, rows,
+                     p.splits);
+  return launched("lse_combine_kernel");
 }
 
 int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, int dtype, int B, int H,

@@ -13,7 +13,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["flash_colreduce", "row_lse2"]
+__all__ = ["flash_colreduce", "flash_colreduce_multi", "row_lse2"]
 
 _DTYPES = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}
 
@@ -55,7 +55,11 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
     return x if ok else x.contiguous()
 
 
-def _launch(query, key, reduction, is_causal, scale, want_out=True):
+def _launch(query, key, kinds, is_causal, scale):
+    """Runs the row kernel once and the column kernel once per entry of `kinds` ('sum' / 'max').
+
+    Returns ([fp32 (B*H, N) per kind], fp32 lse (B*H*M,)).  All device memory comes from torch.
+    """
     b, h, m, d = query.shape
     n = key.shape[2]
     if scale is None:
@@ -64,26 +68,49 @@ def _launch(query, key, reduction, is_causal, scale, want_out=True):
     k = _device_layout(key)
     lib = _lib.load()
     dev = query.device
-    lse = torch.empty((b * h, m), device=dev, dtype=torch.float32)
-    out = torch.empty((b * h, n), device=dev, dtype=torch.float32) if want_out else None
+    # the row statistics, followed by whatever scratch the row kernel wants for this shape
+    nfloat = max(b * h * m, lib.fcr_lse_bytes(b, h, m, n) // 4)
+    lse = torch.empty(nfloat, device=dev, dtype=torch.float32)
+    outs = [torch.empty((b * h, n), device=dev, dtype=torch.float32) for _ in kinds]
     if b * h * m * n == 0:
         lse.fill_(float("-inf"))
-        if want_out:
-            out.zero_()
+        for o in outs:
+            o.zero_()
     else:
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
             common = (_lib.DTYPE_F16 if q.dtype == torch.float16 else _lib.DTYPE_BF16,
                       b, h, m, n, q.shape[3], _lib.strides4(q.stride()), _lib.strides4(k.stride()),
                       float(scale))
-            if want_out:
-                red = _lib.REDUCE_MAX if reduction == "max" else _lib.REDUCE_SUM
-                _lib.check(lib.fcr_colreduce(q.data_ptr(), k.data_ptr(), out.data_ptr(), lse.data_ptr(),
-                                             *common, red, int(bool(is_causal)), stream))
+            causal = int(bool(is_causal))
+            if len(kinds) == 1:
+                red = _lib.REDUCE_MAX if kinds[0] == "max" else _lib.REDUCE_SUM
+                _lib.check(lib.fcr_colreduce(q.data_ptr(), k.data_ptr(), outs[0].data_ptr(), lse.data_ptr(),
+                                             *common, red, causal, stream))
             else:
-                _lib.check(lib.fcr_row_lse(q.data_ptr(), k.data_ptr(), lse.data_ptr(), *common,
-                                           int(bool(is_causal)), stream))
-    return out, lse
+                _lib.check(lib.fcr_row_lse(q.data_ptr(), k.data_ptr(), lse.data_ptr(), *common, causal, stream))
+                for kind, o in zip(kinds, outs):
+                    red = _lib.REDUCE_MAX if kind == "max" else _lib.REDUCE_SUM
+                    _lib.check(lib.fcr_col_reduce(q.data_ptr(), k.data_ptr(), lse.data_ptr(), o.data_ptr(),
+                                                  *common, red, causal, stream))
+    return outs, lse[: b * h * m]
+
+
+def _finish(acc, reduction, query, m, n, is_causal, res_dtype, shared=False):
+    """Cast of the fp32 accumulation and the mean epilogue, as flash.py:308 and 377-385.
+
+    `shared`: the accumulation also feeds other results, so it must not be divided in place."""
+    b, h = query.shape[0], query.shape[1]
+    scores = acc.view(b, h, n).to(res_dtype, copy=shared)
+    if reduction == "mean":
+        # M for keys left of the offset, N-j from the offset on
+        if is_causal:
+            c = max(n - m, 0)
+            scores[..., :c] /= m
+            scores[..., c:] /= torch.arange(n - c, 0, -1, device=query.device)
+        else:
+            scores /= m
+    return scores
 
 
 def flash_colreduce(
@@ -113,19 +140,52 @@ def flash_colreduce(
     if m == 0 and n > 0 and b * h > 0 and reduction == "max":
         raise ValueError("reduction='max' needs at least one query row.")
     if m == 0:
-        scores = torch.zeros((b, h, n), device=query.device, dtype=res_dtype)
+        acc = torch.zeros((b * h, n), device=query.device, dtype=torch.float32)
     else:
-        out, _ = _launch(query, key, reduction, is_causal, scale)
-        scores = out.view(b, h, n).to(res_dtype)
-    if reduction == "mean":
-        # flash.py:377-384: M for keys left of the offset, N-j from the offset on
-        if is_causal:
-            c = max(n - m, 0)
-            scores[..., :c] /= m
-            scores[..., c:] /= torch.arange(n - c, 0, -1, device=query.device)
-        else:
-            scores /= m
-    return scores
+        (acc,), _ = _launch(query, key, ["max" if reduction == "max" else "sum"], is_causal, scale)
+    return _finish(acc, reduction, query, m, n, is_causal, res_dtype)
+
+
+def flash_colreduce_multi(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    reductions,
+    is_causal: bool = False,
+    scale: Optional[float] = None,
+    *,
+    out_dtype: Optional[torch.dtype] = None,
+):
+    """Several reductions of the same attention matrix; returns one (B, H, N) tensor per entry.
+
+    Not in the reference, whose callers ask for one reduction per call and recompute everything
+    (flash.py:311-385).  Here the row statistics are computed once and the column sweep runs once per
+    distinct kind ('sum' and 'mean' share one): 'mean' + 'max' costs three kernels instead of four.
+    Each result equals what flash_colreduce returns for that reduction.
+    """
+    reductions = list(reductions)
+    if not reductions:
+        raise ValueError("reductions must name at least one of 'sum', 'mean', 'max'.")
+    _validate(query, key, reductions[0])
+    for r in reductions[1:]:
+        if r not in ("sum", "mean", "max"):
+            raise ValueError(f"Invalid reduction: {r}. Must be 'sum', 'mean', or 'max'.")
+    b, h, m, _ = query.shape
+    n = key.shape[2]
+    res_dtype = query.dtype if out_dtype is None else out_dtype
+    if m == 0 and n > 0 and b * h > 0 and "max" in reductions:
+        raise ValueError("reduction='max' needs at least one query row.")
+    kinds = []
+    for r in reductions:
+        kind = "max" if r == "max" else "sum"
+        if kind not in kinds:
+            kinds.append(kind)
+    if m == 0:
+        accs = [torch.zeros((b * h, n), device=query.device, dtype=torch.float32) for _ in kinds]
+    else:
+        accs, _ = _launch(query, key, kinds, is_causal, scale)
+    by_kind = dict(zip(kinds, accs))
+    return tuple(_finish(by_kind["max" if r == "max" else "sum"], r, query, m, n, is_causal, res_dtype,
+                         shared=True) for r in reductions)
 
 
 def row_lse2(query: torch.Tensor, key: torch.Tensor, is_causal: bool = False,
@@ -137,5 +197,5 @@ def row_lse2(query: torch.Tensor, key: torch.Tensor, is_causal: bool = False,
     """
     _validate(query, key, None)
     b, h, m, _ = query.shape
-    _, lse = _launch(query, key, None, is_causal, scale, want_out=False)
+    _, lse = _launch(query, key, [], is_causal, scale)
     return lse.view(b, h, m)

@@ -15,7 +15,9 @@
  *     8 <= D <= 128.  (The reference takes any strides, flash.py:292-299; a caller with other
  *     layouts makes a contiguous, zero-padded copy first -- the Python host does.)
  *   - lse is fp32 [B*H, M] contiguous: per query row, log2(sum_j 2^(scale*log2(e)*<q_i,k_j>))
- *     over the keys the row may see.  It is the hand-over between the two kernels.
+ *     over the keys the row may see.  It is the hand-over between the two kernels.  The buffer
+ *     fcr_row_lse / fcr_colreduce write it to must be fcr_lse_bytes(B,H,M,N) long (scratch follows
+ *     the result); fcr_col_reduce only reads the first B*H*M floats.
  *   - out is fp32 [B*H, N] contiguous and is fully overwritten (no zero-fill needed, unlike the
  *     atomically accumulated buffer at flash.py:286).
  *   - causal != 0 applies the right-aligned mask: key j takes part in row i iff
@@ -61,8 +63,12 @@ int fcr_version(void);
 /* Text for the last non-zero return value on the calling thread ("" if none). */
 const char* fcr_last_error(void);
 
-/* Bytes of the lse hand-over buffer for a problem: B*H*M*sizeof(float). */
-size_t fcr_lse_bytes(int B, int H, int M);
+/*
+ * Bytes the lse buffer of fcr_row_lse / fcr_colreduce must have for a problem.  The first
+ * B*H*M floats are the result; for few query rows and many keys the row kernel splits the keys of a
+ * tile over several workgroups and keeps their partial results behind it.  0 for an empty problem.
+ */
+size_t fcr_lse_bytes(int B, int H, int M, int N);
 
 /*
  * First kernel: per-row base-2 log-sum-exp over all visible keys.
@@ -88,7 +94,7 @@ int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, i
 /*
  * Both kernels back to back on one stream: the whole of _flash_colreduce (flash.py:277-308)
  * except the final cast to the input dtype, which stays with the host.  lse_ws is scratch of
- * fcr_lse_bytes(B,H,M) bytes that holds the row statistics on return.
+ * fcr_lse_bytes(B,H,M,N) bytes whose first B*H*M floats hold the row statistics on return.
  */
 int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H,
                   int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],

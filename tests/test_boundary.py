@@ -34,8 +34,10 @@ def test_library_exports_every_declared_symbol():
 def test_version_and_sizes():
     lib = _lib.load()
     assert lib.fcr_version() == 100
-    assert lib.fcr_lse_bytes(2, 3, 5) == 2 * 3 * 5 * 4
-    assert lib.fcr_lse_bytes(-1, 3, 5) == 0
+    assert lib.fcr_lse_bytes(2, 3, 5, 7) == 2 * 3 * 5 * 4
+    assert lib.fcr_lse_bytes(1, 32, 8192, 8192) == 32 * 8192 * 4      # enough row tiles: no scratch
+    assert lib.fcr_lse_bytes(1, 32, 128, 4096) == 32 * 128 * 4 * 17   # 16 key ranges + the result
+    assert lib.fcr_lse_bytes(-1, 3, 5, 7) == 0 and lib.fcr_lse_bytes(1, 3, 0, 7) == 0
 
 
 def _call(lib, fn, **over):

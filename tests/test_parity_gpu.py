@@ -132,6 +132,19 @@ def test_ragged_shapes(m, n, d, causal, dtype):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("b,h,m,n,d", [(1, 4, 40, 5000, 64), (1, 32, 128, 4096, 128), (1, 1, 300, 3001, 128),
+                                       (2, 3, 1, 2048, 32), (1, 2, 257, 1100, 72)])
+def test_few_queries_many_keys(b, h, m, n, d, causal):
+    """Shapes where the row kernel splits the keys of a tile over several workgroups and a second
+    small kernel merges the partial log-sum-exps."""
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=n + m)
+    qd, kd = q.cuda(), k.cuda()
+    got = fca.row_lse2(qd, kd, is_causal=causal).double().cpu()
+    torch.testing.assert_close(got, row_lse2_ref(q, k, causal), rtol=0, atol=3e-4)
+    run_all(q, k, causal, what=f"split b{b} h{h} m{m} n{n} d{d}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
 def test_explicit_and_negative_scale(causal):
     q, k = _inputs.randn_pair(1, 4, 200, 333, 64, seed=21)
     for scale in (0.05, 1.0 / 3.0, -0.125, 0.0):
@@ -220,6 +233,23 @@ def test_output_dtype_and_mean_epilogue():
     s = fca.flash_colreduce(q, k, "sum", True)
     div = torch.cat([torch.full((136,), 64.0), torch.arange(64, 0, -1).float()]).cuda()
     torch.testing.assert_close(out, (s / div.to(torch.bfloat16)), rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_multi_reduction_shares_the_row_pass(causal):
+    q, k = _inputs.randn_pair(2, 3, 300, 450, 64, seed=8, dtype=torch.bfloat16)
+    qd, kd = q.cuda(), k.cuda()
+    outs = fca.flash_colreduce_multi(qd, kd, ["mean", "max", "sum", "mean"], is_causal=causal,
+                                     out_dtype=torch.float32)
+    assert len(outs) == 4
+    for red, got in zip(["mean", "max", "sum", "mean"], outs):
+        one = fca.flash_colreduce(qd, kd, red, is_causal=causal, out_dtype=torch.float32)
+        assert torch.equal(got, one), red
+        check(got, colreduce_ref(q, k, red, causal), red, "multi")
+    with pytest.raises(ValueError, match="Invalid reduction: median"):
+        fca.flash_colreduce_multi(qd, kd, ["sum", "median"])
+    with pytest.raises(ValueError, match="at least one"):
+        fca.flash_colreduce_multi(qd, kd, [])
 
 
 def test_python_errors_on_device():
