@@ -230,7 +230,7 @@ __device__ __forceinline__ void mma_pair(f32x16& n0, f32x16& n1, u32x4 (&f)[KS],
 // Every LDS read is issued a sub-step before its use, every global load a chunk before its store,
 // every LDS store half a chunk before the barrier that publishes it.
 // aux_of(lds, sub) reads what the consumer needs per sub-step besides the scores (the column
-// kernel: -lse of the lane's query); it travels with the fragments so that it too is read before
+// kernel: lse of the lane's query); it travels with the fragments so that it too is read before
 // the barrier that lets other waves overwrite the buffer.
 template <int DT, int KS, bool RESIDENT_IS_KEYS, class StoreF, class LoadF, class AuxF, class ConsumeF>
 __device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[2][KS], char* smem,
@@ -547,11 +547,12 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
   pipelined_sweep<DT, KS, true>(
       t_int, nchunks, kf, smem, kStage, lane, stage_store, stage_load,
       [&](const char* lds, int sub) {
-        return -reinterpret_cast<const float*>(lds + St::kBytes)[sub * 32 + (lane & 31)];
+        return reinterpret_cast<const float*>(lds + St::kBytes)[sub * 32 + (lane & 31)];
       },
-      [&](const f32x16& a0, const f32x16& a1, float nlse) {
-        col_update<false, ISMAX>(a0, p.scale2, nlse, col[0], 0);
-        col_update<false, ISMAX>(a1, p.scale2, nlse, col[1], 0);
+      [&](const f32x16& a0, const f32x16& a1, float lse_q) {
+        // negated inside the fma, so the LDS read above is first waited for a sub-step later
+        col_update<false, ISMAX>(a0, p.scale2, -lse_q, col[0], 0);
+        col_update<false, ISMAX>(a1, p.scale2, -lse_q, col[1], 0);
       });
 
   // Reduce over the 32 query lanes: transpose through LDS, one output key per lane.
