@@ -1,0 +1,110 @@
+"""Latency / peak-memory sweep over the reference's 20 benchmark shapes.
+
+    python -m flash_colreduce_amd.benchmark [--budget SECONDS] [--no-naive] [--out FILE]
+
+Same shapes and method as the reference's harness (benchmarks/run.py:11-92): fp16, H = 32, D = 128,
+reduction = "sum"; per implementation one call, a 10-call calibration, then `iters` warm-up calls and
+`iters` timed calls between device synchronisations; peak memory is torch's max_memory_allocated
+around one call.  `iters = max(int(budget / t_call), 10)`; the reference uses a 10 s budget, the
+default here is 2 s.  Prints a plain-text table (the reference renders the same columns with rich).
+"""
+from __future__ import annotations
+
+import argparse
+import sys
+import time
+
+import torch
+
+from . import flash_colreduce, naive_colreduce
+
+CONFIGS = (
+    [dict(b=b, h=32, m=1024, n=1024, d=128, is_causal=False) for b in (1, 4, 16, 64, 256)]
+    + [dict(b=1, h=32, m=n, n=n, d=128, is_causal=False) for n in (1024, 2048, 4096, 8192, 16384)]
+    + [dict(b=b, h=32, m=64, n=16384, d=128, is_causal=True) for b in (1, 4, 16, 64, 256)]
+    + [dict(b=1, h=32, m=512, n=n, d=128, is_causal=True) for n in (16384, 32768, 65536, 131072, 262144)]
+)
+
+
+def _now() -> float:
+    torch.cuda.synchronize()
+    return time.perf_counter()
+
+
+def measure_latency(fn, budget: float) -> float:
+    fn()
+    t0 = _now()
+    for _ in range(10):
+        fn()
+    per_call = (_now() - t0) / 10
+    iters = max(int(budget / max(per_call, 1e-9)), 10)
+    for _ in range(iters):
+        fn()
+    t0 = _now()
+    for _ in range(iters):
+        fn()
+    return (_now() - t0) / iters * 1e3
+
+
+def measure_memory(fn) -> float:
+    torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    torch.cuda.reset_peak_memory_stats()
+    fn()
+    torch.cuda.synchronize()
+    return torch.cuda.max_memory_allocated() / 2**20
+
+
+def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout):
+    name = torch.cuda.get_device_name(0)
+    print(f"Benchmark results on {name} (fp16, reduction=sum)", file=out)
+    head = (f"{'configuration':<48} {'flash ms':>10} {'naive ms':>10} {'speedup':>8} {'flash MB':>10} "
+            f"{'naive MB':>10} {'mem saving':>10} {'TFLOP/s':>9}")
+    print(head, file=out)
+    print("-" * len(head), file=out)
+    rows = []
+    with torch.inference_mode():
+        for cfg in CONFIGS:
+            b, h, m, n, d, causal = (cfg[k] for k in ("b", "h", "m", "n", "d", "is_causal"))
+            g = torch.Generator(device="cuda").manual_seed(0)
+            q = torch.randn(b, h, m, d, device="cuda", dtype=torch.float16, generator=g)
+            k = torch.randn(b, h, n, d, device="cuda", dtype=torch.float16, generator=g)
+            flash = lambda: flash_colreduce(q, k, reduction="sum", is_causal=causal)  # noqa: E731
+            naive = lambda: naive_colreduce(q, k, reduction="sum", is_causal=causal)  # noqa: E731
+            f_ms, f_mb = measure_latency(flash, budget), measure_memory(flash)
+            n_ms = n_mb = float("nan")
+            if with_naive:
+                try:
+                    n_ms, n_mb = measure_latency(naive, budget), measure_memory(naive)
+                except torch.OutOfMemoryError:
+                    torch.cuda.empty_cache()
+            # visible scores: right-aligned mask hides a triangle of side m-1 when causal
+            visible = m * n - (m * (m - 1) // 2 if causal else 0)
+            tflops = 4.0 * b * h * visible * d / (f_ms * 1e-3) / 1e12
+            label = ",".join(f"{key}={val}" for key, val in cfg.items())
+            print(f"{label:<48} {f_ms:>10.3f} {n_ms:>10.3f} {n_ms / f_ms:>8.2f} {f_mb:>10.1f} {n_mb:>10.1f} "
+                  f"{n_mb / f_mb:>10.2f} {tflops:>9.1f}", file=out, flush=True)
+            rows.append(dict(cfg, flash_ms=f_ms, naive_ms=n_ms, flash_mb=f_mb, naive_mb=n_mb, tflops=tflops))
+            del q, k
+            torch.cuda.empty_cache()
+    return rows
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--budget", type=float, default=2.0, help="seconds of timed calls per implementation")
+    ap.add_argument("--no-naive", action="store_true", help="skip the materialising implementation")
+    ap.add_argument("--out", default=None, help="also write the table to this file")
+    args = ap.parse_args()
+    if not torch.cuda.is_available():
+        raise SystemExit("benchmark needs a GPU")
+    if args.out:
+        with open(args.out, "w") as f:
+            run(args.budget, not args.no_naive, out=f)
+        print(open(args.out).read())
+    else:
+        run(args.budget, not args.no_naive)
+
+
+if __name__ == "__main__":
+    main()
