@@ -65,7 +65,7 @@ def main():
     q_cpu, k_cpu = _inputs.headline()
     q, k = q_cpu.to(dev), k_cpu.to(dev)
     out = torch.empty(B * H, N, device=dev, dtype=torch.float32)
-    lse = torch.empty(lib.fcr_lse_bytes(B, H, M, N) // 4, device=dev, dtype=torch.float32)
+    lse = torch.empty(lib.fcr_lse_bytes(B, H, M, N, D) // 4, device=dev, dtype=torch.float32)
     scale = 1.0 / (D ** 0.5)
     stream = torch.cuda.current_stream(dev).cuda_stream
     common = (_lib.DTYPE_F16, B, H, M, N, D, _lib.strides4(q.stride()), _lib.strides4(k.stride()), scale)

@@ -38,7 +38,7 @@ def _declare(lib):
     lib.fcr_last_error.restype = c.c_char_p
     lib.fcr_last_error.argtypes = []
     lib.fcr_lse_bytes.restype = c.c_size_t
-    lib.fcr_lse_bytes.argtypes = [c.c_int, c.c_int, c.c_int, c.c_int]
+    lib.fcr_lse_bytes.argtypes = [c.c_int, c.c_int, c.c_int, c.c_int, c.c_int]
     lib.fcr_row_lse.restype = c.c_int
     lib.fcr_row_lse.argtypes = [c.c_void_p, c.c_void_p, c.c_void_p] + common + [c.c_int, c.c_void_p]
     lib.fcr_col_reduce.restype = c.c_int

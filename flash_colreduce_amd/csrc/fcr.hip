@@ -33,8 +33,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
-constexpr int kWaveRows = 64;                 // resident rows per wave: two 32-row MFMA blocks
-constexpr int kTileRows = kWaves * kWaveRows; // resident rows per workgroup (eight blocks)
+// Resident 32-row blocks per wave: two while their fragments fit the register file next to the
+// accumulators (D <= 128: 8 k-steps), one for larger D.  A workgroup keeps 4 * 32 * blocks rows.
+__host__ __device__ constexpr int blocks_per_wave(int ksteps) { return ksteps <= 8 ? 2 : 1; }
+__host__ __device__ constexpr int tile_rows(int ksteps) { return kWaves * 32 * blocks_per_wave(ksteps); }
+constexpr int kMaxKSteps = 16;                // D <= 256
 constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row blocks)
 constexpr float kNegInf = -__builtin_inff();
 constexpr float kPosInf = __builtin_inff();
@@ -98,12 +101,14 @@ __device__ __forceinline__ void map_block_split(const Params& p, bool longest_is
   tile = longest_is_last_tile ? p.tiles - 1 - rank : rank;
 }
 
-// A workgroup's 256 resident rows are eight 32-row blocks; wave w keeps blocks w and 7-w.  On a
-// causal diagonal block b has b+1 (rows) or 8-b (columns) visible sub-tiles out of 8, so every wave
-// gets 9 of the 36 and the four waves reach each barrier together.
-__device__ __forceinline__ void wave_blocks(int tile, int wave, int (&rows)[2]) {
-  rows[0] = tile * kTileRows + 32 * wave;
-  rows[1] = tile * kTileRows + 32 * (7 - wave);
+// With two blocks per wave a workgroup's 256 resident rows are eight 32-row blocks and wave w keeps
+// blocks w and 7-w.  On a causal diagonal block b has b+1 (rows) or 8-b (columns) visible sub-tiles
+// out of 8, so every wave gets 9 of the 36 and the four waves reach each barrier together.
+// With one block per wave, wave w keeps block w of four.
+template <int NB>
+__device__ __forceinline__ void wave_blocks(int tile, int wave, int (&rows)[NB]) {
+  rows[0] = tile * (kWaves * 32 * NB) + 32 * wave;
+  if (NB == 2) rows[NB - 1] = tile * (kWaves * 32 * NB) + 32 * (7 - wave);
 }
 
 // Raw buffer view of rows [row0, nrows) of a row-major operand.  Loads through it return zero
@@ -121,15 +126,15 @@ __device__ __forceinline__ u32x4 view_load16(__amdgpu_buffer_rsrc_t v, uint32_t 
   return __builtin_amdgcn_raw_buffer_load_b128(v, (int)byte_off, 0, 0);
 }
 
-// The operand a wave keeps for the whole sweep: two blocks of 32 rows starting at rows[0] and
-// rows[1], as MFMA fragments.  Lane l holds, for k-step ks, the 8 elements
+// The operand a wave keeps for the whole sweep: NB blocks of 32 rows starting at rows[blk], as MFMA
+// fragments.  Lane l holds, for k-step ks, the 8 elements
 // [16*ks + 8*(l/32), +8) of row (l & 31) of a block.
-template <int KS>
-__device__ __forceinline__ void load_resident(u32x4 (&f)[2][KS], const char* base, int64_t row_bytes,
-                                              const int (&rows)[2], int nrows, int dgran, int lane) {
+template <int KS, int NB>
+__device__ __forceinline__ void load_resident(u32x4 (&f)[NB][KS], const char* base, int64_t row_bytes,
+                                              const int (&rows)[NB], int nrows, int dgran, int lane) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int blk = 0; blk < 2; ++blk) {
+  for (int blk = 0; blk < NB; ++blk) {
     const __amdgpu_buffer_rsrc_t view = rows_view(base, row_bytes, rows[blk], nrows);
     const uint32_t roff = (uint32_t)(lane & 31) * (uint32_t)row_bytes;
 #pragma unroll
@@ -195,24 +200,24 @@ struct Stager {
   }
 };
 
-// One sub-step of a sweep: 32 streamed rows (fragments f) against the wave's 64 resident rows, as
-// two independent accumulator chains.  S^T = K * Q^T, so keys are the A operand.  When REFILL, each
+// One sub-step of a sweep: 32 streamed rows (fragments f) against the wave's NB resident blocks, as
+// NB independent accumulator chains.  S^T = K * Q^T, so keys are the A operand.  When REFILL, each
 // fragment register is reloaded for the sub-step after this one as soon as its MFMAs are issued, a
 // whole sub-step ahead of its use.
-template <int DT, int KS, bool RESIDENT_IS_KEYS, bool REFILL>
-__device__ __forceinline__ void mma_pair(f32x16& n0, f32x16& n1, u32x4 (&f)[KS], const u32x4 (&res)[2][KS],
-                                         const char* next_lds, int next_sub, int lane) {
+template <int DT, int KS, int NB, bool RESIDENT_IS_KEYS, bool REFILL>
+__device__ __forceinline__ void mma_blocks(f32x16 (&n)[NB], u32x4 (&f)[KS], const u32x4 (&res)[NB][KS],
+                                           const char* next_lds, int next_sub, int lane) {
   using St = Stager<KS>;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) { n0[r] = 0.f; n1[r] = 0.f; }
+  for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) n[blk][r] = 0.f;
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
-    if (RESIDENT_IS_KEYS) {
-      n0 = mma<DT>(res[0][ks], f[ks], n0);
-      n1 = mma<DT>(res[1][ks], f[ks], n1);
-    } else {
-      n0 = mma<DT>(f[ks], res[0][ks], n0);
-      n1 = mma<DT>(f[ks], res[1][ks], n1);
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk) {
+      if (RESIDENT_IS_KEYS) n[blk] = mma<DT>(res[blk][ks], f[ks], n[blk]);
+      else n[blk] = mma<DT>(f[ks], res[blk][ks], n[blk]);
     }
     if (REFILL) f[ks] = St::frag(next_lds, next_sub, ks, lane);
   }
@@ -232,14 +237,14 @@ __device__ __forceinline__ void mma_pair(f32x16& n0, f32x16& n1, u32x4 (&f)[KS],
 // aux_of(lds, sub) reads what the consumer needs per sub-step besides the scores (the column
 // kernel: lse of the lane's query); it travels with the fragments so that it too is read before
 // the barrier that lets other waves overwrite the buffer.
-template <int DT, int KS, bool RESIDENT_IS_KEYS, class StoreF, class LoadF, class AuxF, class ConsumeF>
-__device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[2][KS], char* smem,
+template <int DT, int KS, int NB, bool RESIDENT_IS_KEYS, class StoreF, class LoadF, class AuxF, class ConsumeF>
+__device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[NB][KS], char* smem,
                                                 int stage_bytes, int lane, StoreF&& stage_store,
                                                 LoadF&& stage_load, AuxF&& aux_of, ConsumeF&& consume) {
   using St = Stager<KS>;
   if (ta >= tb) return;
   u32x4 f[KS];
-  f32x16 p0, p1, n0, n1;
+  f32x16 pa[NB], pb[NB];  // scores of the sub-step being consumed / being produced, swapping roles
   float af, ap, an;
   __syncthreads();
   stage_store(smem + ((ta + 1) & 1) * stage_bytes);
@@ -249,28 +254,26 @@ __device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&re
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) f[ks] = St::frag(lds, 0, ks, lane);
     ap = aux_of(lds, 0);
-    mma_pair<DT, KS, RESIDENT_IS_KEYS, true>(p0, p1, f, res, lds, 1, lane);
+    mma_blocks<DT, KS, NB, RESIDENT_IS_KEYS, true>(pa, f, res, lds, 1, lane);
     af = aux_of(lds, 1);
   }
   for (int t = ta; t + 1 < tb; ++t) {
     const char* nxt = smem + ((t + 1) & 1) * stage_bytes;
     __syncthreads();
     an = af;
-    mma_pair<DT, KS, RESIDENT_IS_KEYS, true>(n0, n1, f, res, nxt, 0, lane);
+    mma_blocks<DT, KS, NB, RESIDENT_IS_KEYS, true>(pb, f, res, nxt, 0, lane);
     af = aux_of(nxt, 0);
-    consume(p0, p1, ap);
-    p0 = n0; p1 = n1; ap = an;
+    consume(pa, ap);
     stage_store(smem + (t & 1) * stage_bytes);
     stage_load(t + 3);
-    an = af;
-    mma_pair<DT, KS, RESIDENT_IS_KEYS, true>(n0, n1, f, res, nxt, 1, lane);
+    ap = af;
+    mma_blocks<DT, KS, NB, RESIDENT_IS_KEYS, true>(pa, f, res, nxt, 1, lane);
     af = aux_of(nxt, 1);
-    consume(p0, p1, ap);
-    p0 = n0; p1 = n1; ap = an;
+    consume(pb, an);
   }
-  mma_pair<DT, KS, RESIDENT_IS_KEYS, false>(n0, n1, f, res, nullptr, 0, lane);
-  consume(p0, p1, ap);
-  consume(n0, n1, af);
+  mma_blocks<DT, KS, NB, RESIDENT_IS_KEYS, false>(pb, f, res, nullptr, 0, lane);
+  consume(pa, ap);
+  consume(pb, af);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -329,18 +332,24 @@ __device__ __forceinline__ void lse_update(const f32x16& acc, float scale2, floa
   else lse_renorm<MASK>(acc, scale2, mref, l, lim);
 }
 
-// Both blocks of a fully visible sub-step; one rarely taken branch at the very end so that the
+// All blocks of a fully visible sub-step; one rarely taken branch at the very end so that the
 // arithmetic above it can be scheduled against the MFMAs of the next sub-step.
-__device__ __forceinline__ void lse_update_pair(const f32x16& a0, const f32x16& a1, float scale2,
-                                                float (&mref)[2], float (&l)[2]) {
-  const float ln0 = lse_fast<false>(a0, scale2, mref[0], l[0], 0);
-  const float ln1 = lse_fast<false>(a1, scale2, mref[1], l[1], 0);
-  if (__builtin_amdgcn_ballot_w64(!(lse_in_range(ln0) && lse_in_range(ln1))) == 0) {
-    l[0] = ln0;
-    l[1] = ln1;
+template <int NB>
+__device__ __forceinline__ void lse_update_blocks(const f32x16 (&a)[NB], float scale2, float (&mref)[NB],
+                                                  float (&l)[NB]) {
+  float ln[NB];
+  bool ok = true;
+#pragma unroll
+  for (int blk = 0; blk < NB; ++blk) {
+    ln[blk] = lse_fast<false>(a[blk], scale2, mref[blk], l[blk], 0);
+    ok = ok && lse_in_range(ln[blk]);
+  }
+  if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk) l[blk] = ln[blk];
   } else {
-    lse_renorm<false>(a0, scale2, mref[0], l[0], 0);
-    lse_renorm<false>(a1, scale2, mref[1], l[1], 0);
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk) lse_renorm<false>(a[blk], scale2, mref[blk], l[blk], 0);
   }
 }
 
@@ -353,6 +362,8 @@ __device__ __forceinline__ float lse_merge(float a, float b) {
 template <int DT, int KS, bool CAUSAL>
 __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   using St = Stager<KS>;
+  constexpr int NB = blocks_per_wave(KS);
+  constexpr int kTileRows = tile_rows(KS);
   __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
   int bh, tile, split;
   map_block_split(p, CAUSAL, bh, tile, split);
@@ -362,10 +373,10 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
   const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
 
-  int q0[2];  // first query of each of this wave's blocks
-  wave_blocks(tile, wave, q0);
-  u32x4 qf[2][KS];
-  load_resident<KS>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
+  int q0[NB];  // first query of each of this wave's blocks
+  wave_blocks<NB>(tile, wave, q0);
+  u32x4 qf[NB][KS];
+  load_resident<KS, NB>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
 
   // Keys [0, kend) matter to this workgroup.  Chunks [0, t_int) are seen in full by every one of
   // its queries and lie inside [0, N): they take the branch-free pipelined sweep.  The rest (the
@@ -378,10 +389,12 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   const int nchunks = min((kend + kChunk - 1) / kChunk, c_begin + per_split);
   const int t_int = min(nchunks, CAUSAL ? min((tile * kTileRows + p.c + 1) / kChunk, p.N / kChunk) : p.N / kChunk);
 
-  float mref[2] = {0.f, 0.f}, l[2] = {0.f, 0.f};
-  int last[2];  // last key a lane's query may see, minus the lane's row offset in a block
+  float mref[NB], l[NB];
+  int last[NB];  // last key a lane's query may see, minus the lane's row offset in a block
 #pragma unroll
-  for (int blk = 0; blk < 2; ++blk) {
+  for (int blk = 0; blk < NB; ++blk) {
+    mref[blk] = 0.f;
+    l[blk] = 0.f;
     const int i = q0[blk] + (lane & 31);
     last[blk] = (CAUSAL ? min(p.N - 1, i + p.c) : p.N - 1) - 4 * (lane >> 5);
   }
@@ -395,10 +408,10 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   stage_store(smem + (c_begin & 1) * St::kBytes);
   stage_load(c_begin + 1);
 
-  pipelined_sweep<DT, KS, false>(
+  pipelined_sweep<DT, KS, NB, false>(
       c_begin, t_int, qf, smem, St::kBytes, lane, stage_store, stage_load,
       [](const char*, int) { return 0.f; },
-      [&](const f32x16& a0, const f32x16& a1, float) { lse_update_pair(a0, a1, p.scale2, mref, l); });
+      [&](const f32x16(&a)[NB], float) { lse_update_blocks<NB>(a, p.scale2, mref, l); });
 
   for (int t = max(t_int, c_begin); t < nchunks; ++t) {
     __syncthreads();  // chunk t published, the other buffer is free
@@ -410,7 +423,7 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
       const int key0 = t * kChunk + sub * 32;
       if (key0 >= p.N) continue;
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
+      for (int blk = 0; blk < NB; ++blk) {
         const int qblk = q0[blk];
         if (CAUSAL && key0 > qblk + 31 + p.c) continue;  // block cannot see this sub-tile
         f32x16 acc = {0};
@@ -424,7 +437,7 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   }
 
 #pragma unroll
-  for (int blk = 0; blk < 2; ++blk) {
+  for (int blk = 0; blk < NB; ++blk) {
     float v = (l[blk] > 0.f) ? mref[blk] + fast_log2(l[blk]) : kNegInf;
     const float o = __shfl_xor(v, 32);
     v = lse_merge(v, o);
@@ -463,8 +476,10 @@ __device__ __forceinline__ void col_update(const f32x16& acc, float scale2, floa
 template <int DT, int KS, bool CAUSAL, bool ISMAX>
 __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p) {
   using St = Stager<KS>;
+  constexpr int NB = blocks_per_wave(KS);
+  constexpr int kTileRows = tile_rows(KS);
   constexpr int kStage = St::kBytes + kChunk * 4;     // rows + their lse
-  constexpr int kRed = kWaves * 32 * 64 * 4;          // end-of-sweep transpose buffer
+  constexpr int kRed = kWaves * NB * 16 * 64 * 4;     // end-of-sweep transpose buffer
   constexpr int kSmem = (2 * kStage > kRed) ? 2 * kStage : kRed;
   __shared__ __attribute__((aligned(16))) char smem[kSmem];
   int bh, tile;
@@ -476,14 +491,14 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
   const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
   const float* lse = p.lse + (int64_t)bh * p.M;
 
-  int k0[2];  // first key of each of this wave's blocks
-  wave_blocks(tile, wave, k0);
-  u32x4 kf[2][KS];
-  load_resident<KS>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
+  int k0[NB];  // first key of each of this wave's blocks
+  wave_blocks<NB>(tile, wave, k0);
+  u32x4 kf[NB][KS];
+  load_resident<KS, NB>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
 
-  f32x16 col[2];
+  f32x16 col[NB];
 #pragma unroll
-  for (int blk = 0; blk < 2; ++blk)
+  for (int blk = 0; blk < NB; ++blk)
 #pragma unroll
     for (int r = 0; r < 16; ++r) col[blk][r] = ISMAX ? kNegInf : 0.f;
 
@@ -530,7 +545,7 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
       if (qs >= p.M) continue;
       const float nlse = -lds_lse[sub * 32 + (lane & 31)];
 #pragma unroll
-      for (int blk = 0; blk < 2; ++blk) {
+      for (int blk = 0; blk < NB; ++blk) {
         const int kblk = k0[blk];
         if (kblk >= p.N) continue;
         if (CAUSAL && kblk > qs + 31 + p.c) continue;  // no query of the sub-tile sees this block
@@ -544,26 +559,26 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
     }
   }
 
-  pipelined_sweep<DT, KS, true>(
+  pipelined_sweep<DT, KS, NB, true>(
       t_int, nchunks, kf, smem, kStage, lane, stage_store, stage_load,
       [&](const char* lds, int sub) {
         return reinterpret_cast<const float*>(lds + St::kBytes)[sub * 32 + (lane & 31)];
       },
-      [&](const f32x16& a0, const f32x16& a1, float lse_q) {
+      [&](const f32x16(&a)[NB], float lse_q) {
         // negated inside the fma, so the LDS read above is first waited for a sub-step later
-        col_update<false, ISMAX>(a0, p.scale2, -lse_q, col[0], 0);
-        col_update<false, ISMAX>(a1, p.scale2, -lse_q, col[1], 0);
+#pragma unroll
+        for (int blk = 0; blk < NB; ++blk) col_update<false, ISMAX>(a[blk], p.scale2, -lse_q, col[blk], 0);
       });
 
   // Reduce over the 32 query lanes: transpose through LDS, one output key per lane.
   __syncthreads();
-  float* red = reinterpret_cast<float*>(smem) + wave * (32 * 64);
+  float* red = reinterpret_cast<float*>(smem) + wave * (NB * 16 * 64);
 #pragma unroll
-  for (int blk = 0; blk < 2; ++blk)
+  for (int blk = 0; blk < NB; ++blk)
 #pragma unroll
     for (int r = 0; r < 16; ++r) red[(blk * 16 + r) * 64 + lane] = col[blk][r];
   __syncthreads();
-  {
+  if ((lane >> 5) < NB) {  // lanes 32.. have no block of their own when a wave keeps one
     const int w = lane & 31;
     const int idx = (lane >> 5) * 16 + (w >> 3) * 4 + (w & 3);
     const float* src = red + idx * 64 + ((w >> 2) & 1) * 32;
@@ -607,10 +622,11 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   if (!q || !k || !qs || !ks) return fail(FCR_E_NULL, "null pointer argument");
   if (dtype != FCR_DTYPE_F16 && dtype != FCR_DTYPE_BF16) return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16 or FCR_DTYPE_BF16");
   if (B < 1 || H < 1 || M < 1 || N < 1) return fail(FCR_E_SHAPE, "B, H, M, N must be >= 1");
-  if (D < 8 || D > 128 || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 128]");
+  if (D < 8 || D > 16 * kMaxKSteps || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 256]");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
-  const int64_t tiles = ((by_keys ? N : M) + kTileRows - 1) / kTileRows;
+  const int trows = tile_rows((D + 15) / 16);
+  const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
   if (bh * tiles > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
   if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
   int rc = check_strides(q, qs, "q");
@@ -638,8 +654,9 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
 // Key ranges per row tile in the row kernel.  One sweep per workgroup when there is at least one
 // workgroup per CU; otherwise the keys of a tile are split so that about two per CU run, each
 // keeping at least four 64-key chunks.
-int row_splits(int B, int H, int M, int N) {
-  const int64_t wgs = (int64_t)B * H * ((M + kTileRows - 1) / kTileRows);
+int row_splits(int B, int H, int M, int N, int D) {
+  const int trows = tile_rows((D + 15) / 16);
+  const int64_t wgs = (int64_t)B * H * ((M + trows - 1) / trows);
   const int64_t chunks = (N + kChunk - 1) / kChunk;
   if (wgs >= 256 || chunks < 16) return 1;
   int64_t s = 512 / wgs;
@@ -683,7 +700,15 @@ void launch_col(const Params& p, bool causal, bool ismax, hipStream_t s) {
     case 5: CALL(DT, 5); break;                            \
     case 6: CALL(DT, 6); break;                            \
     case 7: CALL(DT, 7); break;                            \
-    default: CALL(DT, 8); break;                           \
+    case 8: CALL(DT, 8); break;                            \
+    case 9: CALL(DT, 9); break;                            \
+    case 10: CALL(DT, 10); break;                          \
+    case 11: CALL(DT, 11); break;                          \
+    case 12: CALL(DT, 12); break;                          \
+    case 13: CALL(DT, 13); break;                          \
+    case 14: CALL(DT, 14); break;                          \
+    case 15: CALL(DT, 15); break;                          \
+    default: CALL(DT, 16); break;                          \
   }
 
 }  // namespace
@@ -694,9 +719,9 @@ int fcr_version(void) { return FCR_VERSION; }
 
 const char* fcr_last_error(void) { return g_err; }
 
-size_t fcr_lse_bytes(int B, int H, int M, int N) {
-  if (B < 1 || H < 1 || M < 1 || N < 1) return 0;
-  const int splits = row_splits(B, H, M, N);
+size_t fcr_lse_bytes(int B, int H, int M, int N, int D) {
+  if (B < 1 || H < 1 || M < 1 || N < 1 || D < 1) return 0;
+  const int splits = row_splits(B, H, M, N, D);
   const size_t rows = (size_t)B * (size_t)H * (size_t)M;
   return rows * sizeof(float) * (splits > 1 ? 1 + (size_t)splits : 1);
 }
@@ -709,7 +734,7 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
   int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, false);
   if (rc) return rc;
   p.lse = lse;
-  p.splits = row_splits(B, H, M, N);
+  p.splits = row_splits(B, H, M, N, D);
   p.part = lse + (int64_t)B * H * M;  // only touched when splits > 1 (see fcr_lse_bytes)
   p.total *= p.splits;
   const int ksteps = (D + 15) / 16;

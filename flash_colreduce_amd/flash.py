@@ -36,8 +36,8 @@ def _validate(query: torch.Tensor, key: torch.Tensor, reduction: Optional[str]):
         )
     if query.device != key.device:
         raise ValueError("Query and key tensors must be on the same device.")
-    if query.shape[3] > 128:
-        raise ValueError(f"Head dimension must be <= 128. Got {query.shape[3]}.")
+    if query.shape[3] > 256:
+        raise ValueError(f"Head dimension must be <= 256. Got {query.shape[3]}.")
 
 
 def _device_layout(x: torch.Tensor) -> torch.Tensor:
@@ -69,7 +69,7 @@ def _launch(query, key, kinds, is_causal, scale):
     lib = _lib.load()
     dev = query.device
     # the row statistics, followed by whatever scratch the row kernel wants for this shape
-    nfloat = max(b * h * m, lib.fcr_lse_bytes(b, h, m, n) // 4)
+    nfloat = max(b * h * m, lib.fcr_lse_bytes(b, h, m, n, q.shape[3]) // 4)
     lse = torch.empty(nfloat, device=dev, dtype=torch.float32)
     outs = [torch.empty((b * h, n), device=dev, dtype=torch.float32) for _ in kinds]
     if b * h * m * n == 0:

@@ -12,11 +12,11 @@
  *   - q is [B,H,M,D], k is [B,H,N,D], 16-bit elements (dtype below).  Strides are in ELEMENTS,
  *     order (batch, head, row, d); the d stride must be 1, row/head/batch strides must be
  *     multiples of 8 elements and the base pointers 16-byte aligned, D a multiple of 8 and
- *     8 <= D <= 128.  (The reference takes any strides, flash.py:292-299; a caller with other
+ *     8 <= D <= 256.  (The reference takes any strides, flash.py:292-299; a caller with other
  *     layouts makes a contiguous, zero-padded copy first -- the Python host does.)
  *   - lse is fp32 [B*H, M] contiguous: per query row, log2(sum_j 2^(scale*log2(e)*<q_i,k_j>))
  *     over the keys the row may see.  It is the hand-over between the two kernels.  The buffer
- *     fcr_row_lse / fcr_colreduce write it to must be fcr_lse_bytes(B,H,M,N) long (scratch follows
+ *     fcr_row_lse / fcr_colreduce write it to must be fcr_lse_bytes(B,H,M,N,D) long (scratch follows
  *     the result); fcr_col_reduce only reads the first B*H*M floats.
  *   - out is fp32 [B*H, N] contiguous and is fully overwritten (no zero-fill needed, unlike the
  *     atomically accumulated buffer at flash.py:286).
@@ -52,7 +52,7 @@ extern "C" {
 /* argument errors */
 #define FCR_E_NULL -1      /* a required pointer is NULL */
 #define FCR_E_DTYPE -2     /* dtype is not FCR_DTYPE_* */
-#define FCR_E_SHAPE -3     /* B,H,M,N < 1, D outside [8,128] or not a multiple of 8, sizes overflow */
+#define FCR_E_SHAPE -3     /* B,H,M,N < 1, D outside [8,256] or not a multiple of 8, sizes overflow */
 #define FCR_E_STRIDE -4    /* d stride != 1 or a stride / base pointer breaks 16-byte alignment */
 #define FCR_E_REDUCTION -5 /* reduction is not FCR_REDUCE_* */
 #define FCR_E_SCALE -6     /* scale is not finite */
@@ -68,7 +68,7 @@ const char* fcr_last_error(void);
  * B*H*M floats are the result; for few query rows and many keys the row kernel splits the keys of a
  * tile over several workgroups and keeps their partial results behind it.  0 for an empty problem.
  */
-size_t fcr_lse_bytes(int B, int H, int M, int N);
+size_t fcr_lse_bytes(int B, int H, int M, int N, int D);
 
 /*
  * First kernel: per-row base-2 log-sum-exp over all visible keys.
@@ -94,7 +94,7 @@ int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, i
 /*
  * Both kernels back to back on one stream: the whole of _flash_colreduce (flash.py:277-308)
  * except the final cast to the input dtype, which stays with the host.  lse_ws is scratch of
- * fcr_lse_bytes(B,H,M,N) bytes whose first B*H*M floats hold the row statistics on return.
+ * fcr_lse_bytes(B,H,M,N,D) bytes whose first B*H*M floats hold the row statistics on return.
  */
 int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H,
                   int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],

@@ -34,10 +34,10 @@ def test_library_exports_every_declared_symbol():
 def test_version_and_sizes():
     lib = _lib.load()
     assert lib.fcr_version() == 100
-    assert lib.fcr_lse_bytes(2, 3, 5, 7) == 2 * 3 * 5 * 4
-    assert lib.fcr_lse_bytes(1, 32, 8192, 8192) == 32 * 8192 * 4      # enough row tiles: no scratch
-    assert lib.fcr_lse_bytes(1, 32, 128, 4096) == 32 * 128 * 4 * 17   # 16 key ranges + the result
-    assert lib.fcr_lse_bytes(-1, 3, 5, 7) == 0 and lib.fcr_lse_bytes(1, 3, 0, 7) == 0
+    assert lib.fcr_lse_bytes(2, 3, 5, 7, 64) == 2 * 3 * 5 * 4
+    assert lib.fcr_lse_bytes(1, 32, 8192, 8192, 128) == 32 * 8192 * 4      # enough row tiles: no scratch
+    assert lib.fcr_lse_bytes(1, 32, 128, 4096, 128) == 32 * 128 * 4 * 17   # 16 key ranges + the result
+    assert lib.fcr_lse_bytes(-1, 3, 5, 7, 8) == 0 and lib.fcr_lse_bytes(1, 3, 0, 7, 8) == 0
 
 
 def _call(lib, fn, **over):
@@ -62,7 +62,7 @@ def test_c_abi_rejects_bad_arguments_without_a_device(fn):
         (dict(q=None), -1), (dict(k=None), -1), (dict(lse=None), -1), (dict(qs=None), -1),
         (dict(dtype=2), -2), (dict(dtype=-1), -2),
         (dict(B=0), -3), (dict(M=0), -3), (dict(N=-4), -3), (dict(D=0), -3), (dict(D=12), -3),
-        (dict(D=136), -3), (dict(M=(1 << 30) + 1), -3),
+        (dict(D=264), -3), (dict(M=(1 << 30) + 1), -3),
         (dict(qs=(512, 512, 64, 2)), -4), (dict(ks=(512, 512, 60, 1)), -4), (dict(q=18), -4),
         (dict(ks=(512, -512, 64, 1)), -4),
         (dict(scale=float("inf")), -6), (dict(scale=float("nan")), -6),

@@ -131,6 +131,16 @@ def test_ragged_shapes(m, n, d, causal, dtype):
     run_all(q, k, causal, what=f"m{m} n{n} d{d} {dtype}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n,d", [(300, 420, 136), (257, 129, 192), (130, 1000, 256), (64, 64, 200),
+                                   (1, 700, 250), (520, 520, 144)])
+def test_head_dims_above_128(m, n, d, causal, dtype):
+    """D in (128, 256]: one resident 32-row block per wave, 128-row tiles."""
+    q, k = _inputs.randn_pair(1, 3, m, n, d, seed=d + m, dtype=dtype)
+    run_all(q, k, causal, what=f"m{m} n{n} d{d} {dtype}")
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("b,h,m,n,d", [(1, 4, 40, 5000, 64), (1, 32, 128, 4096, 128), (1, 1, 300, 3001, 128),
                                        (2, 3, 1, 2048, 32), (1, 2, 257, 1100, 72)])
