@@ -595,6 +595,29 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
 }
 
 // ---------------------------------------------------------------------------------------------
+// fp32 operands.  x = hi + lo with hi = fp16(x), lo = fp16(x - hi) carries 22 bits of x.  Packing
+// queries as [hi | hi | lo] and keys as [hi | lo | hi] along d makes the fp16 kernels compute
+// q_hi.k_hi + q_hi.k_lo + q_lo.k_hi, the product to about 2^-22 (the lo.lo term is dropped), with fp32
+// accumulation.  With terms == 1 only [hi] is written (both operands rounded to fp16).
+// dst rows are terms * dpad halves, each segment zero padded from D to dpad.
+__global__ __launch_bounds__(256) void pack_f32_kernel(const float* __restrict__ src, _Float16* __restrict__ dst,
+                                                       int64_t rows, int D, int dpad, int terms, int is_key) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= rows * dpad) return;
+  const int64_t row = idx / dpad;
+  const int d = (int)(idx - row * dpad);
+  const float x = (d < D) ? src[row * D + d] : 0.f;
+  const _Float16 hi = (_Float16)x;
+  _Float16* out = dst + row * (int64_t)(terms * dpad) + d;
+  out[0] = hi;
+  if (terms == 3) {
+    const _Float16 lo = (_Float16)(x - (float)hi);
+    out[dpad] = is_key ? lo : hi;
+    out[2 * dpad] = is_key ? hi : lo;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 thread_local char g_err[256] = "";
 
 int fail(int code, const char* what) {
@@ -769,6 +792,20 @@ int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, i
   else { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL) }
 #undef FCR_CALL_COL
   return launched("col_reduce_kernel");
+}
+
+int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, int is_key, void* stream) {
+  if (!src || !dst) return fail(FCR_E_NULL, "null pointer argument");
+  if (rows < 1 || D < 1) return fail(FCR_E_SHAPE, "rows and D must be >= 1");
+  if (terms != 1 && terms != 3) return fail(FCR_E_SHAPE, "terms must be 1 or 3");
+  const int dpad = (D + 7) / 8 * 8;
+  if (terms * dpad > 16 * kMaxKSteps) return fail(FCR_E_SHAPE, "terms * D (padded to 8) must be <= 256");
+  const int64_t n = rows * dpad;
+  if ((n + 255) / 256 > 0x7fffffffll) return fail(FCR_E_SHAPE, "too many elements");
+  hipLaunchKernelGGL(pack_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), src, static_cast<_Float16*>(dst), rows, D, dpad, terms,
+                     is_key != 0);
+  return launched("pack_f32_kernel");
 }
 
 int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H, int M,

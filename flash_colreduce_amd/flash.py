@@ -29,9 +29,9 @@ def _validate(query: torch.Tensor, key: torch.Tensor, reduction: Optional[str]):
         )
     if reduction is not None and reduction not in ("sum", "mean", "max"):
         raise ValueError(f"Invalid reduction: {reduction}. Must be 'sum', 'mean', or 'max'.")
-    if query.dtype != key.dtype or query.dtype not in _DTYPES:
+    if query.dtype != key.dtype or (query.dtype not in _DTYPES and query.dtype != torch.float32):
         raise ValueError(
-            f"Query and key tensors must both be float16 or bfloat16. "
+            f"Query and key tensors must both be float16, bfloat16 or float32. "
             f"Got query dtype: {query.dtype}, key dtype: {key.dtype}."
         )
     if query.device != key.device:
@@ -55,6 +55,24 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
     return x if ok else x.contiguous()
 
 
+def _pack_f32(x: torch.Tensor, is_key: bool) -> torch.Tensor:
+    """fp32 operand -> the fp16 layout the kernels take (see fcr_pack_f32 in include/fcr.h).
+
+    Three fp16 segments [hi|hi|lo] / [hi|lo|hi] when they fit in 256 columns (D <= 80): the product
+    is then good to about 2^-22.  Larger D is rounded to fp16 once, which is what the reference's
+    tl.dot does to fp32 operands on its hardware (TF32 has fewer mantissa bits than fp16)."""
+    b, h, r, d = x.shape
+    dpad = (d + 7) // 8 * 8
+    terms = 3 if 3 * dpad <= 256 else 1
+    src = x.contiguous()
+    dst = torch.empty((b, h, r, terms * dpad), device=x.device, dtype=torch.float16)
+    if dst.numel():
+        with torch.cuda.device(x.device):
+            _lib.check(_lib.load().fcr_pack_f32(src.data_ptr(), dst.data_ptr(), b * h * r, d, terms,
+                                                int(is_key), torch.cuda.current_stream(x.device).cuda_stream))
+    return dst
+
+
 def _launch(query, key, kinds, is_causal, scale):
     """Runs the row kernel once and the column kernel once per entry of `kinds` ('sum' / 'max').
 
@@ -64,8 +82,11 @@ def _launch(query, key, kinds, is_causal, scale):
     n = key.shape[2]
     if scale is None:
         scale = 1 / math.sqrt(d)  # the unpadded D (flash.py:366-367)
-    q = _device_layout(query)
-    k = _device_layout(key)
+    if query.dtype == torch.float32:
+        q, k = _pack_f32(query, False), _pack_f32(key, True)
+    else:
+        q = _device_layout(query)
+        k = _device_layout(key)
     lib = _lib.load()
     dev = query.device
     # the row statistics, followed by whatever scratch the row kernel wants for this shape
@@ -124,8 +145,8 @@ def flash_colreduce(
 ) -> torch.Tensor:
     """Per-key sum / mean / max over queries of softmax(Q K^T * scale), shape (B, H, N).
 
-    Args follow the reference (flash.py:311-352): query (B,H,M,D), key (B,H,N,D), fp16 or bf16 on
-    the GPU; `is_causal` applies the right-aligned mask (key j visible to query i iff
+    Args follow the reference (flash.py:311-352): query (B,H,M,D), key (B,H,N,D), fp16, bf16 or
+    fp32 on the GPU, D <= 256; `is_causal` applies the right-aligned mask (key j visible to query i iff
     j <= i + max(N-M, 0)); `scale` defaults to 1/sqrt(D).
 
     `out_dtype` (keyword only, not in the reference) selects the result dtype.  None reproduces

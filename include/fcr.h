@@ -92,6 +92,17 @@ int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, i
                    void* stream);
 
 /*
+ * fp32 operands: packs a contiguous fp32 [rows, D] into the fp16 [rows, terms * Dp] (Dp = D rounded up
+ * to 8, zero padded) that the kernels above take with D' = terms * Dp and dtype FCR_DTYPE_F16.
+ * terms = 3 writes [hi | hi | lo] for queries (is_key = 0) and [hi | lo | hi] for keys (is_key != 0),
+ * hi = fp16(x), lo = fp16(x - hi): the kernels then see q.k to about 2^-22.  terms = 1 writes [hi].
+ * terms * Dp must be <= 256; values beyond the fp16 range overflow.  scale must be passed explicitly
+ * to the kernels (1/sqrt(D) of the original D).  The reference feeds fp32 straight to tl.dot
+ * (flash.py:59,108), which on its hardware rounds both operands to TF32.
+ */
+int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, int is_key, void* stream);
+
+/*
  * Both kernels back to back on one stream: the whole of _flash_colreduce (flash.py:277-308)
  * except the final cast to the input dtype, which stays with the host.  lse_ws is scratch of
  * fcr_lse_bytes(B,H,M,N,D) bytes whose first B*H*M floats hold the row statistics on return.

@@ -77,6 +77,16 @@ def test_c_abi_rejects_bad_arguments_without_a_device(fn):
     assert e.value.code == -3 and "multiple of 8" in str(e.value)
 
 
+def test_pack_f32_rejects_bad_arguments_without_a_device():
+    lib = _lib.load()
+    assert lib.fcr_pack_f32(None, 16, 4, 8, 3, 0, None) == -1
+    assert lib.fcr_pack_f32(16, None, 4, 8, 3, 0, None) == -1
+    assert lib.fcr_pack_f32(16, 32, 0, 8, 3, 0, None) == -3
+    assert lib.fcr_pack_f32(16, 32, 4, 8, 2, 0, None) == -3      # terms must be 1 or 3
+    assert lib.fcr_pack_f32(16, 32, 4, 88, 3, 0, None) == -3     # 3 * 88 > 256
+    assert lib.fcr_pack_f32(16, 32, 4, 264, 1, 0, None) == -3
+
+
 def test_python_entry_validation_matches_reference_messages():
     q = torch.zeros(1, 2, 4, 8, dtype=torch.float16)
     k = torch.zeros(1, 2, 6, 8, dtype=torch.float16)

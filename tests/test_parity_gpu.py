@@ -67,6 +67,37 @@ def test_config1_rounded_to_fp16():
     run_all(q.half(), k.half(), False, what="config1")
 
 
+def test_config1_fp32():
+    """Config 1 as given: fp32 operands.  D = 64 fits the three-segment fp16 split, so the device
+    result is good far beyond the metric's tolerance; 1e-4 would fail with a single fp16 rounding."""
+    q, k = _inputs.config1()
+    qd, kd = q.cuda(), k.cuda()
+    for red in REDUCTIONS:
+        got = fca.flash_colreduce(qd, kd, red)
+        assert got.dtype == torch.float32 and got.shape == (1, 2, 256)
+        want = colreduce_ref(q, k, red, compute_dtype=torch.float64).float()
+        check(got, want, red, "config1 fp32")
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-7)
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n,d", [(100, 260, 20), (257, 300, 80), (64, 500, 128), (130, 140, 200)])
+def test_fp32_operands(m, n, d, causal):
+    """fp32 inputs: split into fp16 hi/lo segments for D <= 80 (near-fp32 products), rounded to
+    fp16 once above that (as accurate as the TF32 rounding the reference's tl.dot applies)."""
+    q, k = _inputs.randn_pair(2, 2, m, n, d, seed=d, dtype=torch.float32)
+    qd, kd = q.cuda(), k.cuda()
+    for red in REDUCTIONS:
+        got = fca.flash_colreduce(qd, kd, red, is_causal=causal, scale=0.11)
+        want = colreduce_ref(q, k, red, causal, scale=0.11, compute_dtype=torch.float64).float()
+        assert got.dtype == torch.float32
+        if d <= 80:
+            check(got, want, red, f"fp32 d{d}")
+            torch.testing.assert_close(got.cpu(), want, rtol=1e-4, atol=1e-7)
+        else:
+            torch.testing.assert_close(got.cpu(), want, rtol=5e-3, atol=1e-5)
+
+
 def test_config2():
     q, k = _inputs.config2()
     run_all(q, k, False, what="config2")
@@ -269,8 +300,10 @@ def test_python_errors_on_device():
         fca.flash_colreduce(q, k, "median")
     with pytest.raises(ValueError, match="same batch size, number of heads, and head dimension"):
         fca.flash_colreduce(q, k[:, :1], "sum")
-    with pytest.raises(ValueError, match="float16 or bfloat16"):
-        fca.flash_colreduce(q.float(), k.float(), "sum")
+    with pytest.raises(ValueError, match="float16, bfloat16 or float32"):
+        fca.flash_colreduce(q.double(), k.double(), "sum")
+    with pytest.raises(ValueError, match="float16, bfloat16 or float32"):
+        fca.flash_colreduce(q.float(), k, "sum")
     # zero queries see no key: every column is 1/N
     out = fca.flash_colreduce(q, k, "max", out_dtype=torch.float32)
     torch.testing.assert_close(out, torch.full((1, 2, 6), 1 / 6, device="cuda"))
