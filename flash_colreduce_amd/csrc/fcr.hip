@@ -48,7 +48,8 @@ struct Params {
   float* lse;        // [BH, M]
   float* part;       // [splits, BH, M] partial lse of key ranges when splits > 1
   int splits;        // key ranges per row tile in the row kernel (1 = whole sweep in one workgroup)
-  float* out;        // [BH, N]
+  float* out;        // [BH, N]: column sums (or the only result)
+  float* out2;       // [BH, N]: column maxima when one sweep produces both
   int64_t q_sb, q_sh, q_sr;  // strides in BYTES: batch, head, row
   int64_t k_sb, k_sh, k_sr;
   int H, M, N;
@@ -461,23 +462,33 @@ __global__ __launch_bounds__(256) void lse_combine_kernel(const float* __restric
 }
 
 // ---------------------------------------------------------------------------------------------
-template <bool MASK, bool ISMAX>
-__device__ __forceinline__ void col_update(const f32x16& acc, float scale2, float nlse, f32x16& col,
-                                           int lim) {
+// What a column sweep produces.
+constexpr int kModeSum = 0, kModeMax = 1, kModeBoth = 2;
+
+// x = s*scale2 - lse is the base-2 log of the probability.  Sums add 2^x; maxima track x itself and
+// exponentiate once at the end of the sweep (2^x is monotone), so a max-only sweep has no exp.
+template <bool MASK, int MODE>
+__device__ __forceinline__ void col_update(const f32x16& acc, float scale2, float nlse, f32x16& csum,
+                                           f32x16& cmax, int lim) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     float x = fmaf(acc[r], scale2, nlse);
     if (MASK) x = (reg_row(r) <= lim) ? x : kNegInf;
-    if (ISMAX) col[r] = fmaxf(col[r], x);
-    else col[r] += fast_exp2(x);
+    if (MODE != kModeSum) cmax[r] = fmaxf(cmax[r], x);
+    if (MODE != kModeMax) csum[r] += fast_exp2(x);
   }
 }
 
-template <int DT, int KS, bool CAUSAL, bool ISMAX>
+// MODE both keeps two sets of column registers, so a wave then holds one block of keys instead of two.
+__host__ __device__ constexpr int col_blocks_per_wave(int ksteps, int mode) {
+  return mode == kModeBoth ? 1 : blocks_per_wave(ksteps);
+}
+
+template <int DT, int KS, bool CAUSAL, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p) {
   using St = Stager<KS>;
-  constexpr int NB = blocks_per_wave(KS);
-  constexpr int kTileRows = tile_rows(KS);
+  constexpr int NB = col_blocks_per_wave(KS, MODE);
+  constexpr int kTileRows = kWaves * 32 * NB;
   constexpr int kStage = St::kBytes + kChunk * 4;     // rows + their lse
   constexpr int kRed = kWaves * NB * 16 * 64 * 4;     // end-of-sweep transpose buffer
   constexpr int kSmem = (2 * kStage > kRed) ? 2 * kStage : kRed;
@@ -496,11 +507,14 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
   u32x4 kf[NB][KS];
   load_resident<KS, NB>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
 
-  f32x16 col[NB];
+  f32x16 csum[NB], cmax[NB];  // the set a MODE does not use is never touched and costs no registers
 #pragma unroll
   for (int blk = 0; blk < NB; ++blk)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) col[blk][r] = ISMAX ? kNegInf : 0.f;
+    for (int r = 0; r < 16; ++r) {
+      csum[blk][r] = 0.f;
+      cmax[blk][r] = kNegInf;
+    }
 
   // Query chunks [t0, nchunks) can see keys of this tile.  From chunk t_int on every query sees
   // all of them: those chunks take the branch-free pipelined sweep (rows past M carry lse = +inf
@@ -553,8 +567,8 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) acc = mma<DT>(kf[blk][ks], St::frag(lds, sub, ks, lane), acc);
         const bool need_mask = CAUSAL && (kblk + 31 > qs + p.c);
-        if (need_mask) col_update<true, ISMAX>(acc, p.scale2, nlse, col[blk], lim_lane + qs - kblk);
-        else col_update<false, ISMAX>(acc, p.scale2, nlse, col[blk], 0);
+        if (need_mask) col_update<true, MODE>(acc, p.scale2, nlse, csum[blk], cmax[blk], lim_lane + qs - kblk);
+        else col_update<false, MODE>(acc, p.scale2, nlse, csum[blk], cmax[blk], 0);
       }
     }
   }
@@ -567,30 +581,45 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
       [&](const f32x16(&a)[NB], float lse_q) {
         // negated inside the fma, so the LDS read above is first waited for a sub-step later
 #pragma unroll
-        for (int blk = 0; blk < NB; ++blk) col_update<false, ISMAX>(a[blk], p.scale2, -lse_q, col[blk], 0);
+        for (int blk = 0; blk < NB; ++blk)
+          col_update<false, MODE>(a[blk], p.scale2, -lse_q, csum[blk], cmax[blk], 0);
       });
 
   // Reduce over the 32 query lanes: transpose through LDS, one output key per lane.
-  __syncthreads();
   float* red = reinterpret_cast<float*>(smem) + wave * (NB * 16 * 64);
+  const int w = lane & 31;
+  const int idx = (lane >> 5) * 16 + (w >> 3) * 4 + (w & 3);
+  const float* src = red + idx * 64 + ((w >> 2) & 1) * 32;
+  const int key = k0[(lane >> 5) < NB ? (lane >> 5) : 0] + w;
+  const bool writer = ((lane >> 5) < NB) && key < p.N;  // lanes 32.. idle when a wave keeps one block
+  if (MODE != kModeMax) {
+    __syncthreads();
 #pragma unroll
-  for (int blk = 0; blk < NB; ++blk)
+    for (int blk = 0; blk < NB; ++blk)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) red[(blk * 16 + r) * 64 + lane] = col[blk][r];
-  __syncthreads();
-  if ((lane >> 5) < NB) {  // lanes 32.. have no block of their own when a wave keeps one
-    const int w = lane & 31;
-    const int idx = (lane >> 5) * 16 + (w >> 3) * 4 + (w & 3);
-    const float* src = red + idx * 64 + ((w >> 2) & 1) * 32;
-    float v = ISMAX ? kNegInf : 0.f;
+      for (int r = 0; r < 16; ++r) red[(blk * 16 + r) * 64 + lane] = csum[blk][r];
+    __syncthreads();
+    if ((lane >> 5) < NB) {
+      float v = 0.f;
 #pragma unroll 8
-    for (int j = 0; j < 32; ++j) {
-      const float x = src[(j + lane) & 31];
-      v = ISMAX ? fmaxf(v, x) : v + x;
+      for (int j = 0; j < 32; ++j) v += src[(j + lane) & 31];
+      if (writer) p.out[(int64_t)bh * p.N + key] = v;
     }
-    if (ISMAX) v = fast_exp2(v);
-    const int key = k0[lane >> 5] + w;
-    if (key < p.N) p.out[(int64_t)bh * p.N + key] = v;
+  }
+  if (MODE != kModeSum) {
+    __syncthreads();
+#pragma unroll
+    for (int blk = 0; blk < NB; ++blk)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) red[(blk * 16 + r) * 64 + lane] = cmax[blk][r];
+    __syncthreads();
+    if ((lane >> 5) < NB) {
+      float v = kNegInf;
+#pragma unroll 8
+      for (int j = 0; j < 32; ++j) v = fmaxf(v, src[(j + lane) & 31]);
+      float* dst = (MODE == kModeBoth) ? p.out2 : p.out;
+      if (writer) dst[(int64_t)bh * p.N + key] = fast_exp2(v);
+    }
   }
 }
 
@@ -641,14 +670,14 @@ int check_strides(const void* ptr, const int64_t s[4], const char* name) {
 }
 
 int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H, int M, int N, int D,
-                const int64_t qs[4], const int64_t ks[4], float scale, bool by_keys) {
+                const int64_t qs[4], const int64_t ks[4], float scale, bool by_keys, int col_mode = kModeSum) {
   if (!q || !k || !qs || !ks) return fail(FCR_E_NULL, "null pointer argument");
   if (dtype != FCR_DTYPE_F16 && dtype != FCR_DTYPE_BF16) return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16 or FCR_DTYPE_BF16");
   if (B < 1 || H < 1 || M < 1 || N < 1) return fail(FCR_E_SHAPE, "B, H, M, N must be >= 1");
   if (D < 8 || D > 16 * kMaxKSteps || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 256]");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
-  const int trows = tile_rows((D + 15) / 16);
+  const int trows = by_keys ? kWaves * 32 * col_blocks_per_wave((D + 15) / 16, col_mode) : tile_rows((D + 15) / 16);
   const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
   if (bh * tiles > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
   if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
@@ -669,6 +698,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   p.total = (int)(bh * tiles);
   p.lse = nullptr;
   p.out = nullptr;
+  p.out2 = nullptr;
   p.part = nullptr;
   p.splits = 1;
   return 0;
@@ -702,16 +732,18 @@ void launch_lse(const Params& p, bool causal, hipStream_t s) {
   else hipLaunchKernelGGL((row_lse_kernel<DT, KS, false>), grid, block, 0, s, p);
 }
 
-template <int DT, int KS>
-void launch_col(const Params& p, bool causal, bool ismax, hipStream_t s) {
+template <int DT, int KS, int MODE>
+void launch_col_mode(const Params& p, bool causal, hipStream_t s) {
   const dim3 grid(p.total), block(kThreads);
-  if (causal) {
-    if (ismax) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, true>), grid, block, 0, s, p);
-    else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, false>), grid, block, 0, s, p);
-  } else {
-    if (ismax) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, true>), grid, block, 0, s, p);
-    else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, false>), grid, block, 0, s, p);
-  }
+  if (causal) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, MODE>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, MODE>), grid, block, 0, s, p);
+}
+
+template <int DT, int KS>
+void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
+  if (mode == kModeSum) launch_col_mode<DT, KS, kModeSum>(p, causal, s);
+  else if (mode == kModeMax) launch_col_mode<DT, KS, kModeMax>(p, causal, s);
+  else launch_col_mode<DT, KS, kModeBoth>(p, causal, s);
 }
 
 #define FCR_DISPATCH_KS(DT, ksteps, CALL)                  \
@@ -774,24 +806,41 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
   return launched("lse_combine_kernel");
 }
 
-int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, int dtype, int B, int H,
-                   int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
-                   float scale, int reduction, int causal, void* stream) {
+namespace {
+int col_reduce_any(const void* q, const void* k, const float* lse, float* out, float* out2, int mode, int dtype,
+                   int B, int H, int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
+                   float scale, int causal, void* stream) {
   Params p;
-  if (!lse || !out) return fail(FCR_E_NULL, "null pointer argument");
-  if (reduction != FCR_REDUCE_SUM && reduction != FCR_REDUCE_MAX)
-    return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM or FCR_REDUCE_MAX");
-  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true);
+  if (!lse || !out || (mode == kModeBoth && !out2)) return fail(FCR_E_NULL, "null pointer argument");
+  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true, mode);
   if (rc) return rc;
   p.lse = const_cast<float*>(lse);
   p.out = out;
+  p.out2 = out2;
   const int ksteps = (D + 15) / 16;
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal != 0, reduction == FCR_REDUCE_MAX, s)
+#define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal != 0, mode, s)
   if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_COL) }
   else { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL) }
 #undef FCR_CALL_COL
   return launched("col_reduce_kernel");
+}
+}  // namespace
+
+int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, int dtype, int B, int H,
+                   int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
+                   float scale, int reduction, int causal, void* stream) {
+  if (reduction != FCR_REDUCE_SUM && reduction != FCR_REDUCE_MAX)
+    return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM or FCR_REDUCE_MAX");
+  return col_reduce_any(q, k, lse, out, nullptr, reduction == FCR_REDUCE_MAX ? kModeMax : kModeSum, dtype, B, H, M,
+                        N, D, q_strides, k_strides, scale, causal, stream);
+}
+
+int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float* out_sum, float* out_max,
+                           int dtype, int B, int H, int M, int N, int D, const int64_t q_strides[4],
+                           const int64_t k_strides[4], float scale, int causal, void* stream) {
+  return col_reduce_any(q, k, lse, out_sum, out_max, kModeBoth, dtype, B, H, M, N, D, q_strides, k_strides, scale,
+                        causal, stream);
 }
 
 int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, int is_key, void* stream) {

@@ -92,6 +92,14 @@ int fcr_col_reduce(const void* q, const void* k, const float* lse, float* out, i
                    void* stream);
 
 /*
+ * Second kernel producing the column sums and the column maxima from ONE sweep (the reference needs two
+ * full calls for that, flash.py:311-385 once per reduction).  out_sum and out_max are fp32 [B*H, N].
+ */
+int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float* out_sum, float* out_max,
+                           int dtype, int B, int H, int M, int N, int D, const int64_t q_strides[4],
+                           const int64_t k_strides[4], float scale, int causal, void* stream);
+
+/*
  * fp32 operands: packs a contiguous fp32 [rows, D] into the fp16 [rows, terms * Dp] (Dp = D rounded up
  * to 8, zero padded) that the kernels above take with D' = terms * Dp and dtype FCR_DTYPE_F16.
  * terms = 3 writes [hi | hi | lo] for queries (is_key = 0) and [hi | lo | hi] for keys (is_key != 0),
