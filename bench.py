@@ -150,7 +150,7 @@ def main():
                   "causal B1 H32 M=N=8192 d128 fp16",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "fp16 MFMA, fp32 accumulate and softmax", "data": "synthetic",
+        "dtype": "fp16", "accumulate": "fp32", "data": "synthetic",
         "config": {"workload": "causal B=1 H=32 M=N=8192 D=128 fp16, reduction=sum, seed 0 N(0,1)",
                    "flop_per_call": flop_call, "frac_of_fp16_dense_peak": value / PEAK_FP16_DENSE_TFLOPS},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "parity": parity,
