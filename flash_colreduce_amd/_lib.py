@@ -46,6 +46,8 @@ def _declare(lib):
                                    [c.c_int, c.c_int, c.c_void_p])
     lib.fcr_col_reduce_sum_max.restype = c.c_int
     lib.fcr_col_reduce_sum_max.argtypes = ([c.c_void_p] * 5 + common + [c.c_int, c.c_void_p])
+    lib.fcr_topk_mask.restype = c.c_int
+    lib.fcr_topk_mask.argtypes = [c.c_void_p, c.c_void_p, c.c_void_p, c.c_int64, c.c_int, c.c_int, c.c_void_p]
     lib.fcr_pack_f32.restype = c.c_int
     lib.fcr_pack_f32.argtypes = [c.c_void_p, c.c_void_p, c.c_int64, c.c_int, c.c_int, c.c_int, c.c_void_p]
     lib.fcr_colreduce.restype = c.c_int

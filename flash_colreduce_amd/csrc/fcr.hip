@@ -647,6 +647,85 @@ __global__ __launch_bounds__(256) void pack_f32_kernel(const float* __restrict__
 }
 
 // ---------------------------------------------------------------------------------------------
+// Keep-mask of the k largest scores of every row (what a pruning caller does with the reduced
+// columns).  One workgroup per row: an 8-bit-digit radix select over the order-preserving integer
+// image of the floats finds the k-th largest value in four counting passes, a last pass writes the
+// mask; elements equal to the threshold are kept from the lowest index up until k are kept.
+__device__ __forceinline__ uint32_t order_key(float x) {
+  uint32_t b = __builtin_bit_cast(uint32_t, x);
+  if (b == 0x80000000u) b = 0u;  // -0 and +0 are one value
+  return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);  // monotone in x for all non-NaN floats
+}
+
+__global__ __launch_bounds__(256) void topk_mask_kernel(const float* __restrict__ scores, uint8_t* __restrict__ mask,
+                                                        float* __restrict__ threshold, int N, int k) {
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t sh_prefix, sh_need, sh_ties, sh_running;
+  __shared__ uint32_t wave_eq[4];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* s = scores + (int64_t)blockIdx.x * N;
+  uint8_t* m = mask + (int64_t)blockIdx.x * N;
+  uint32_t prefix = 0, decided = 0, need = (uint32_t)min(k, N);
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    hist[tid] = 0;
+    __syncthreads();
+    for (int j = tid; j < N; j += 256) {
+      const uint32_t u = order_key(s[j]);
+      if ((u & decided) == prefix) atomicAdd(&hist[(u >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    if (tid == 0) {
+      uint32_t above = 0;
+      int d = 255;
+      for (; d > 0; --d) {
+        if (above + hist[d] >= need) break;
+        above += hist[d];
+      }
+      sh_prefix = prefix | ((uint32_t)d << shift);
+      sh_need = need - above;  // how many of the elements with this digit are still wanted
+      sh_ties = hist[d];
+    }
+    __syncthreads();
+    prefix = sh_prefix;
+    need = sh_need;
+    decided |= 0xffu << shift;
+    __syncthreads();
+  }
+  // prefix is now the key of the k-th largest element; `need` of the sh_ties elements equal to it are kept
+  const bool ordered = sh_ties != need;
+  if (tid == 0) {
+    sh_running = 0;
+    if (threshold) {
+      const uint32_t b = (prefix & 0x80000000u) ? (prefix ^ 0x80000000u) : ~prefix;
+      threshold[blockIdx.x] = __builtin_bit_cast(float, b);
+    }
+  }
+  __syncthreads();
+  for (int base = 0; base < N; base += 256) {
+    const int j = base + tid;
+    const uint32_t u = (j < N) ? order_key(s[j]) : 0u;
+    const bool eq = (j < N) && (u == prefix) && (k > 0);
+    bool keep = (j < N) && (u > prefix) && (k > 0);
+    if (!ordered) {
+      keep = keep || eq;
+    } else {  // wave-uniform: rank the ties by index
+      const uint64_t ballot = __builtin_amdgcn_ballot_w64(eq);
+      if (lane == 0) wave_eq[wave] = (uint32_t)__builtin_popcountll(ballot);
+      __syncthreads();
+      uint32_t before = sh_running;
+      for (int w = 0; w < wave; ++w) before += wave_eq[w];
+      before += (uint32_t)__builtin_popcountll(ballot & ((1ull << lane) - 1ull));
+      keep = keep || (eq && before < need);
+      __syncthreads();
+      if (tid == 0) sh_running += wave_eq[0] + wave_eq[1] + wave_eq[2] + wave_eq[3];
+      __syncthreads();
+    }
+    if (j < N) m[j] = keep ? 1 : 0;
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 thread_local char g_err[256] = "";
 
 int fail(int code, const char* what) {
@@ -841,6 +920,14 @@ int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float
                            const int64_t k_strides[4], float scale, int causal, void* stream) {
   return col_reduce_any(q, k, lse, out_sum, out_max, kModeBoth, dtype, B, H, M, N, D, q_strides, k_strides, scale,
                         causal, stream);
+}
+
+int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream) {
+  if (!scores || !mask) return fail(FCR_E_NULL, "null pointer argument");
+  if (rows < 1 || rows > 0x7fffffffll || N < 1) return fail(FCR_E_SHAPE, "rows must be in [1, 2^31) and N >= 1");
+  hipLaunchKernelGGL(topk_mask_kernel, dim3((unsigned)rows), dim3(256), 0, static_cast<hipStream_t>(stream), scores,
+                     mask, threshold, N, k);
+  return launched("topk_mask_kernel");
 }
 
 int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, int is_key, void* stream) {

@@ -13,7 +13,7 @@ import torch
 
 from . import _lib
 
-__all__ = ["flash_colreduce", "flash_colreduce_multi", "row_lse2"]
+__all__ = ["flash_colreduce", "flash_colreduce_multi", "row_lse2", "topk_keep_mask"]
 
 _DTYPES = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}
 
@@ -227,3 +227,26 @@ def row_lse2(query: torch.Tensor, key: torch.Tensor, is_causal: bool = False,
     b, h, m, _ = query.shape
     _, lse = _launch(query, key, [], is_causal, scale)
     return lse.view(b, h, m)
+
+
+def topk_keep_mask(scores: torch.Tensor, k: int, return_threshold: bool = False):
+    """Boolean mask of the k largest entries along the last dimension (ties: lower index wins).
+
+    The step a pruning caller takes on the (B, H, N) result of flash_colreduce; not part of the
+    reference's package.  `scores` must be a float32 GPU tensor; the result has its shape.
+    With return_threshold also returns the k-th largest value per row, shape scores.shape[:-1].
+    """
+    if not scores.is_cuda:
+        raise ValueError("scores must be on CUDA device.")
+    if scores.dtype != torch.float32 or scores.dim() < 1:
+        raise ValueError(f"scores must be a float32 tensor with at least one dimension. Got {scores.dtype}.")
+    s = scores.contiguous()
+    n = s.shape[-1]
+    rows = s.numel() // n if n else 0
+    mask = torch.zeros(s.shape, device=s.device, dtype=torch.bool)
+    thr = torch.empty(s.shape[:-1], device=s.device, dtype=torch.float32) if return_threshold else None
+    if rows > 0 and n > 0:
+        with torch.cuda.device(s.device):
+            _lib.check(_lib.load().fcr_topk_mask(s.data_ptr(), mask.data_ptr(), thr.data_ptr() if thr is not None else None,
+                                                 rows, n, int(k), torch.cuda.current_stream(s.device).cuda_stream))
+    return (mask, thr) if return_threshold else mask

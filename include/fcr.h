@@ -100,6 +100,15 @@ int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float
                            const int64_t k_strides[4], float scale, int causal, void* stream);
 
 /*
+ * Keep-mask of the k largest of every row of a contiguous fp32 [rows, N] (e.g. the [B*H, N] result of
+ * the calls above): mask[r, j] = 1 for exactly min(max(k,0), N) columns of row r, 0 elsewhere; among
+ * equal values the lower column wins.  threshold (optional, may be NULL) receives the k-th largest
+ * value of each row.  No counterpart in the reference: it is the step its pruning callers take on
+ * the reduced columns (README.md:9).  NaNs are not ordered.
+ */
+int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream);
+
+/*
  * fp32 operands: packs a contiguous fp32 [rows, D] into the fp16 [rows, terms * Dp] (Dp = D rounded up
  * to 8, zero padded) that the kernels above take with D' = terms * Dp and dtype FCR_DTYPE_F16.
  * terms = 3 writes [hi | hi | lo] for queries (is_key = 0) and [hi | lo | hi] for keys (is_key != 0),

@@ -55,6 +55,7 @@ __all__ = [
     "colreduce_bruteforce",
     "colreduce_ref",
     "row_lse2_ref",
+    "topk_mask_ref",
 ]
 
 
@@ -191,3 +192,19 @@ def row_lse2_ref(q: torch.Tensor, k: torch.Tensor, is_causal: bool = False,
                     s = s.masked_fill(cols > rows + c, -math.inf)
                 out[b, h, row0:row0 + qb.shape[0]] = torch.logsumexp(s * math.log(2.0), dim=-1) / math.log(2.0)
     return out
+
+
+def topk_mask_ref(scores, k: int) -> np.ndarray:
+    """Keep-mask of the k largest entries of every row of a 2-D array; among equal values the lower
+    column wins.  Pinned by its defining properties (tests/test_oracle.py::test_topk_mask_ref): exactly
+    min(max(k,0),N) kept, every kept value >= every dropped one, kept ties precede dropped ties.
+    The reference has no such function; its callers do this step themselves (README.md:9)."""
+    a = np.asarray(scores)
+    rows, n = a.shape
+    kk = min(max(int(k), 0), n)
+    mask = np.zeros((rows, n), dtype=bool)
+    cols = np.arange(n)
+    for r in range(rows):
+        order = np.lexsort((cols, -a[r].astype(np.float64)))  # by value descending, then column ascending
+        mask[r, order[:kk]] = True
+    return mask

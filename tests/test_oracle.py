@@ -180,6 +180,26 @@ def test_row_lse2(causal):
         np.testing.assert_allclose(lse[:, :, i].numpy(), want.numpy(), rtol=1e-12)
 
 
+def test_topk_mask_ref():
+    from oracle.colreduce_oracle import topk_mask_ref
+    a = np.array([[0.5, 0.25, 0.5, 0.125, 0.5], [-1.0, 3.0, 0.0, -0.0, 2.0]])
+    np.testing.assert_array_equal(topk_mask_ref(a, 2), [[1, 0, 1, 0, 0], [0, 1, 0, 0, 1]])
+    np.testing.assert_array_equal(topk_mask_ref(a, 4), [[1, 1, 1, 0, 1], [0, 1, 1, 1, 1]])
+    assert not topk_mask_ref(a, 0).any() and topk_mask_ref(a, 9).all() and not topk_mask_ref(a, -3).any()
+    rng = np.random.default_rng(0)
+    b = rng.integers(0, 6, size=(7, 40)).astype(np.float32)  # many ties
+    for k in (1, 5, 17, 39):
+        m = topk_mask_ref(b, k)
+        assert (m.sum(1) == k).all()
+        for r in range(7):
+            kept, dropped = b[r][m[r]], b[r][~m[r]]
+            assert kept.min() >= dropped.max()
+            t = kept.min()
+            tie_cols = np.nonzero(b[r] == t)[0]
+            kept_ties = [c for c in tie_cols if m[r, c]]
+            assert kept_ties == list(tie_cols[:len(kept_ties)])
+
+
 def test_bad_reduction():
     q, k = _rand(1, 1, 2, 2, 2)
     with pytest.raises(ValueError, match="Invalid reduction"):

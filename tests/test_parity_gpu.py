@@ -311,6 +311,36 @@ def test_sum_and_max_from_one_sweep(m, n, d, causal, dtype):
     check(mean, colreduce_ref(q, k, "mean", causal), "mean", "fused")
 
 
+@pytest.mark.parametrize("n,k", [(1, 1), (5, 2), (256, 100), (257, 256), (1000, 0), (1000, 1000), (1000, 1500),
+                                 (4099, 1024), (32768, 8192)])
+def test_topk_keep_mask(n, k):
+    from oracle.colreduce_oracle import topk_mask_ref
+    g = torch.Generator().manual_seed(n + k)
+    vals = torch.rand(6, n, generator=g)
+    vals[1] = (vals[1] * 8).floor() / 8          # heavy ties
+    vals[2] = 0.25                                # all equal
+    vals[3] = -vals[3]                            # negatives
+    vals[4, ::3] = 0.0
+    vals[4, 1::3] = -0.0
+    mask, thr = fca.topk_keep_mask(vals.cuda().view(2, 3, n), k, return_threshold=True)
+    assert mask.dtype == torch.bool and mask.shape == (2, 3, n) and thr.shape == (2, 3)
+    want = topk_mask_ref(vals.numpy(), k)
+    assert (mask.view(6, n).cpu().numpy() == want).all()
+    if 0 < k <= n:
+        kth = torch.sort(vals, dim=1, descending=True).values[:, k - 1]
+        assert torch.equal(thr.view(6).cpu(), kth)
+
+
+def test_topk_on_reduced_columns():
+    from oracle.colreduce_oracle import topk_mask_ref
+    q, k = _inputs.config4(heads=4, n=2048)
+    s = fca.flash_colreduce(q.cuda(), k.cuda(), "sum", is_causal=True, out_dtype=torch.float32)
+    mask = fca.topk_keep_mask(s, 512)
+    assert (mask.sum(-1) == 512).all()
+    assert (mask.view(4, 2048).cpu().numpy() == topk_mask_ref(s.view(4, 2048).cpu().numpy(), 512)).all()
+    assert mask[..., 0].all()   # the sink column is always kept
+
+
 def test_python_errors_on_device():
     q = torch.zeros(1, 2, 4, 8, dtype=torch.float16, device="cuda")
     k = torch.zeros(1, 2, 6, 8, dtype=torch.float16, device="cuda")
