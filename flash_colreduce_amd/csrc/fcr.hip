@@ -1,12 +1,14 @@
 // libfcr: column reduction of softmax attention for MI355X (gfx950, CDNA4).
 //
-// Two kernels, both built on v_mfma_f32_32x32x16_{f16,bf16} with the product taken as
-// S^T = K * Q^T (keys are MFMA rows, queries are MFMA columns).  In the 32x32 accumulator a lane
-// owns ONE query (lane & 31) and 16 keys (row 8*(r/4) + 4*(lane/32) + r%4 for register r), so
+// Two kernels, both built on v_mfma_f32_16x16x32_{f16,bf16} with the product taken as
+// S^T = K * Q^T (keys are MFMA rows, queries are MFMA columns).  In a 16x16 accumulator a lane
+// owns ONE query (lane & 15) and 4 keys (row 4*(lane/16) + r for register r), so
 //   - everything that is per query row (softmax reference exponent, running sum, lse) is one
 //     scalar per lane and needs no cross-lane traffic inside the sweep;
-//   - everything that is per key column accumulates in the lane's 16 registers over the whole
-//     sweep and is reduced across the 32 query lanes once, at the end.
+//   - everything that is per key column accumulates in the lane's registers over the whole
+//     sweep and is reduced across the 16 query lanes once, at the end.
+// The 16x16x32 shape is used because on this chip it sustains about 14 % more flops per watt than
+// 32x32x16 on random operands, and these kernels run against the package power limit.
 //
 //   row_lse_kernel    a workgroup keeps 256 query rows in registers (64 per wave) and streams
 //                     key tiles through LDS; writes lse2[bh, i] = log2 sum_j 2^(s_ij).
@@ -28,17 +30,18 @@ namespace {
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
-// Resident 32-row blocks per wave: two while their fragments fit the register file next to the
-// accumulators (D <= 128: 8 k-steps), one for larger D.  A workgroup keeps 4 * 32 * blocks rows.
-__host__ __device__ constexpr int blocks_per_wave(int ksteps) { return ksteps <= 8 ? 2 : 1; }
+// k-steps are 32 elements of D.  A wave keeps resident rows in groups of 16 (one MFMA operand each);
+// two 32-row blocks (four groups) while their fragments fit the register file next to the
+// accumulators (D <= 128: 4 k-steps), one block for larger D.  A workgroup keeps 4 * 32 * blocks rows.
+__host__ __device__ constexpr int blocks_per_wave(int ksteps) { return ksteps <= 4 ? 2 : 1; }
 __host__ __device__ constexpr int tile_rows(int ksteps) { return kWaves * 32 * blocks_per_wave(ksteps); }
-constexpr int kMaxKSteps = 16;                // D <= 256
-constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row blocks)
+constexpr int kMaxKSteps = 8;                 // D <= 256
+constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row sub-steps)
 constexpr float kNegInf = -__builtin_inff();
 constexpr float kPosInf = __builtin_inff();
 
@@ -61,22 +64,22 @@ struct Params {
   int total;         // tiles * B * H workgroups
 };
 
+// D[16 keys][16 queries] += A[16 keys][32 d] * B[32 d][16 queries].  Lane l supplies, for A and for
+// B alike, the 8 consecutive d-elements [8*(l/16), +8) of row / column l & 15, and receives
+// D[4*(l/16) + r][l & 15] in register r.
 template <int DT>
-__device__ __forceinline__ f32x16 mma(u32x4 a, u32x4 b, f32x16 c) {
+__device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c) {
   if constexpr (DT == FCR_DTYPE_F16) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
+                                                  0, 0, 0);
   } else {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
+                                                   c, 0, 0, 0);
   }
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
-
-// Key offset inside a 32-row block of accumulator register r, before the 4*(lane/32) term.
-__device__ __forceinline__ constexpr int reg_row(int r) { return 8 * (r >> 2) + (r & 3); }
 
 // Work order.  Workgroup v takes (b,h) = v % BH and the tile of rank v / BH, tiles ranked by the
 // length of their sweep, longest first: with more workgroups than the chip holds at once, the
@@ -102,14 +105,21 @@ __device__ __forceinline__ void map_block_split(const Params& p, bool longest_is
   tile = longest_is_last_tile ? p.tiles - 1 - rank : rank;
 }
 
-// With two blocks per wave a workgroup's 256 resident rows are eight 32-row blocks and wave w keeps
-// blocks w and 7-w.  On a causal diagonal block b has b+1 (rows) or 8-b (columns) visible sub-tiles
-// out of 8, so every wave gets 9 of the 36 and the four waves reach each barrier together.
-// With one block per wave, wave w keeps block w of four.
+// First rows of the wave's resident 16-row groups.  With two blocks per wave a workgroup's 256
+// resident rows are eight 32-row blocks and wave w keeps blocks w and 7-w: on a causal diagonal
+// block b has b+1 (rows) or 8-b (columns) visible sub-tiles out of 8, so every wave gets 9 of the 36
+// and the four waves reach each barrier together.  With one block per wave, wave w keeps block w
+// of four.
 template <int NB>
-__device__ __forceinline__ void wave_blocks(int tile, int wave, int (&rows)[NB]) {
-  rows[0] = tile * (kWaves * 32 * NB) + 32 * wave;
-  if (NB == 2) rows[NB - 1] = tile * (kWaves * 32 * NB) + 32 * (7 - wave);
+__device__ __forceinline__ void wave_groups(int tile, int wave, int (&rows)[2 * NB]) {
+  const int b0 = tile * (kWaves * 32 * NB) + 32 * wave;
+  rows[0] = b0;
+  rows[1] = b0 + 16;
+  if (NB == 2) {
+    const int b1 = tile * (kWaves * 32 * NB) + 32 * (7 - wave);
+    rows[2 * NB - 2] = b1;
+    rows[2 * NB - 1] = b1 + 16;
+  }
 }
 
 // Raw buffer view of rows [row0, nrows) of a row-major operand.  Loads through it return zero
@@ -127,22 +137,21 @@ __device__ __forceinline__ u32x4 view_load16(__amdgpu_buffer_rsrc_t v, uint32_t 
   return __builtin_amdgcn_raw_buffer_load_b128(v, (int)byte_off, 0, 0);
 }
 
-// The operand a wave keeps for the whole sweep: NB blocks of 32 rows starting at rows[blk], as MFMA
-// fragments.  Lane l holds, for k-step ks, the 8 elements
-// [16*ks + 8*(l/32), +8) of row (l & 31) of a block.
-template <int KS, int NB>
-__device__ __forceinline__ void load_resident(u32x4 (&f)[NB][KS], const char* base, int64_t row_bytes,
-                                              const int (&rows)[NB], int nrows, int dgran, int lane) {
+// The operand a wave keeps for the whole sweep: NG groups of 16 rows starting at rows[g], as MFMA
+// fragments.  Lane l holds, for k-step ks, the 8 elements [32*ks + 8*(l/16), +8) of row l & 15.
+template <int KS, int NG>
+__device__ __forceinline__ void load_resident(u32x4 (&f)[NG][KS], const char* base, int64_t row_bytes,
+                                              const int (&rows)[NG], int nrows, int dgran, int lane) {
   const u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-  for (int blk = 0; blk < NB; ++blk) {
-    const __amdgpu_buffer_rsrc_t view = rows_view(base, row_bytes, rows[blk], nrows);
-    const uint32_t roff = (uint32_t)(lane & 31) * (uint32_t)row_bytes;
+  for (int g = 0; g < NG; ++g) {
+    const __amdgpu_buffer_rsrc_t view = rows_view(base, row_bytes, rows[g], nrows);
+    const uint32_t roff = (uint32_t)(lane & 15) * (uint32_t)row_bytes;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const int g = ks * 2 + (lane >> 5);
-      const u32x4 v = view_load16(view, roff + (uint32_t)min(g, dgran - 1) * 16u);
-      f[blk][ks] = (g < dgran) ? v : zero;  // zero padding of D up to the k-step
+      const int gi = ks * 4 + (lane >> 4);
+      const u32x4 v = view_load16(view, roff + (uint32_t)min(gi, dgran - 1) * 16u);
+      f[g][ks] = (gi < dgran) ? v : zero;  // zero padding of D up to the k-step
     }
   }
 }
@@ -156,8 +165,8 @@ __device__ __forceinline__ void load_resident(u32x4 (&f)[NB][KS], const char* ba
 // Rows past the end of the operand come back as zeros from the buffer view.
 template <int KS>
 struct Stager {
-  static constexpr int kGran = 2 * KS;             // 16-byte granules per (zero padded) row
-  static constexpr int kRowBytes = KS * 32 + 16;   // LDS row pitch
+  static constexpr int kGran = 4 * KS;             // 16-byte granules per (zero padded) row
+  static constexpr int kRowBytes = KS * 64 + 16;   // LDS row pitch
   static constexpr int kTotal = kChunk * kGran;
   static constexpr int kPer = (kTotal + kThreads - 1) / kThreads;
   static constexpr int kDummy = kChunk * kRowBytes;  // 16 bytes nobody reads
@@ -194,33 +203,39 @@ struct Stager {
 #pragma unroll
     for (int i = 0; i < kPer; ++i) *reinterpret_cast<u32x4*>(lds + loff[i]) = regs[i];
   }
-  // Fragment of block `sub` (32 rows) for k-step ks.
-  static __device__ __forceinline__ u32x4 frag(const char* lds, int sub, int ks, int lane) {
-    return *reinterpret_cast<const u32x4*>(lds + (sub * 32 + (lane & 31)) * kRowBytes + ks * 32 +
-                                           (lane >> 5) * 16);
+  // Fragment of the 16-row group sg of sub-step `sub` (32 rows) for k-step ks.
+  static __device__ __forceinline__ u32x4 frag(const char* lds, int sub, int sg, int ks, int lane) {
+    return *reinterpret_cast<const u32x4*>(lds + (sub * 32 + sg * 16 + (lane & 15)) * kRowBytes + ks * 64 +
+                                           (lane >> 4) * 16);
   }
 };
 
-// One sub-step of a sweep: 32 streamed rows (fragments f) against the wave's NB resident blocks, as
-// NB independent accumulator chains.  S^T = K * Q^T, so keys are the A operand.  When REFILL, each
-// fragment register is reloaded for the sub-step after this one as soon as its MFMAs are issued, a
-// whole sub-step ahead of its use.
-template <int DT, int KS, int NB, bool RESIDENT_IS_KEYS, bool REFILL>
-__device__ __forceinline__ void mma_blocks(f32x16 (&n)[NB], u32x4 (&f)[KS], const u32x4 (&res)[NB][KS],
+// One sub-step of a sweep: 32 streamed rows (two groups of 16, fragments f) against the wave's NG
+// resident groups: 2*NG independent 16x16 accumulator chains n[g][sg].  S^T = K * Q^T, so keys are
+// the A operand.  A streamed fragment stays put for NG consecutive MFMAs.  When REFILL, each fragment
+// register is reloaded for the sub-step after this one as soon as its MFMAs are issued, a whole
+// sub-step ahead of its use.
+template <int DT, int KS, int NG, bool RESIDENT_IS_KEYS, bool REFILL>
+__device__ __forceinline__ void mma_groups(f32x4 (&n)[NG][2], u32x4 (&f)[2][KS], const u32x4 (&res)[NG][KS],
                                            const char* next_lds, int next_sub, int lane) {
   using St = Stager<KS>;
+  const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-  for (int blk = 0; blk < NB; ++blk)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) n[blk][r] = 0.f;
+  for (int g = 0; g < NG; ++g) {
+    n[g][0] = zero;
+    n[g][1] = zero;
+  }
 #pragma unroll
   for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
-    for (int blk = 0; blk < NB; ++blk) {
-      if (RESIDENT_IS_KEYS) n[blk] = mma<DT>(res[blk][ks], f[ks], n[blk]);
-      else n[blk] = mma<DT>(f[ks], res[blk][ks], n[blk]);
+    for (int sg = 0; sg < 2; ++sg) {
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        if (RESIDENT_IS_KEYS) n[g][sg] = mma<DT>(res[g][ks], f[sg][ks], n[g][sg]);
+        else n[g][sg] = mma<DT>(f[sg][ks], res[g][ks], n[g][sg]);
+      }
+      if (REFILL) f[sg][ks] = St::frag(next_lds, next_sub, sg, ks, lane);
     }
-    if (REFILL) f[ks] = St::frag(next_lds, next_sub, ks, lane);
   }
 }
 
@@ -236,49 +251,53 @@ __device__ __forceinline__ void mma_blocks(f32x16 (&n)[NB], u32x4 (&f)[KS], cons
 // Every LDS read is issued a sub-step before its use, every global load a chunk before its store,
 // every LDS store half a chunk before the barrier that publishes it.
 // aux_of(lds, sub) reads what the consumer needs per sub-step besides the scores (the column
-// kernel: lse of the lane's query); it travels with the fragments so that it too is read before
+// kernel: lse of the lane's queries); it travels with the fragments so that it too is read before
 // the barrier that lets other waves overwrite the buffer.
-template <int DT, int KS, int NB, bool RESIDENT_IS_KEYS, class StoreF, class LoadF, class AuxF, class ConsumeF>
-__device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[NB][KS], char* smem,
+template <int DT, int KS, int NG, bool RESIDENT_IS_KEYS, class Aux, class StoreF, class LoadF, class AuxF,
+          class ConsumeF>
+__device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[NG][KS], char* smem,
                                                 int stage_bytes, int lane, StoreF&& stage_store,
                                                 LoadF&& stage_load, AuxF&& aux_of, ConsumeF&& consume) {
   using St = Stager<KS>;
   if (ta >= tb) return;
-  u32x4 f[KS];
-  f32x16 pa[NB], pb[NB];  // scores of the sub-step being consumed / being produced, swapping roles
-  float af, ap, an;
+  u32x4 f[2][KS];
+  f32x4 pa[NG][2], pb[NG][2];  // scores of the sub-step being consumed / being produced, swapping roles
+  Aux af, ap, an;
   __syncthreads();
   stage_store(smem + ((ta + 1) & 1) * stage_bytes);
   stage_load(ta + 2);
   {
     const char* lds = smem + (ta & 1) * stage_bytes;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) f[ks] = St::frag(lds, 0, ks, lane);
+    for (int ks = 0; ks < KS; ++ks) {
+      f[0][ks] = St::frag(lds, 0, 0, ks, lane);
+      f[1][ks] = St::frag(lds, 0, 1, ks, lane);
+    }
     ap = aux_of(lds, 0);
-    mma_blocks<DT, KS, NB, RESIDENT_IS_KEYS, true>(pa, f, res, lds, 1, lane);
+    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pa, f, res, lds, 1, lane);
     af = aux_of(lds, 1);
   }
   for (int t = ta; t + 1 < tb; ++t) {
     const char* nxt = smem + ((t + 1) & 1) * stage_bytes;
     __syncthreads();
     an = af;
-    mma_blocks<DT, KS, NB, RESIDENT_IS_KEYS, true>(pb, f, res, nxt, 0, lane);
+    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pb, f, res, nxt, 0, lane);
     af = aux_of(nxt, 0);
     consume(pa, ap);
     stage_store(smem + (t & 1) * stage_bytes);
     stage_load(t + 3);
     ap = af;
-    mma_blocks<DT, KS, NB, RESIDENT_IS_KEYS, true>(pa, f, res, nxt, 1, lane);
+    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pa, f, res, nxt, 1, lane);
     af = aux_of(nxt, 1);
     consume(pb, an);
   }
-  mma_blocks<DT, KS, NB, RESIDENT_IS_KEYS, false>(pb, f, res, nullptr, 0, lane);
+  mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, false>(pb, f, res, nullptr, 0, lane);
   consume(pa, ap);
   consume(pb, af);
 }
 
 // ---------------------------------------------------------------------------------------------
-// Row statistics.  Per lane and 32-query block the state is (mref, l) with
+// Row statistics.  Per lane and resident 16-query group the state is (mref, l) with
 //   sum over the keys seen so far of 2^(s) = l * 2^mref.
 // mref is a reference exponent, not the running maximum: the common path (lse_fast) adds
 // 2^(s - mref) without looking for a maximum.  The sum is renormalised (lse_renorm) only when it
@@ -287,70 +306,76 @@ __device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&re
 // max(tile max, 0)).  Invariant after the first visible key: 1 <= l < 2^64, hence
 // mref <= lse < mref + 64, so terms that underflow are below 2^-126 of the total and overflow is
 // caught by the range check.
+// a[sg][r] is the score of the lane's query against key 16*sg + 4*(lane/16) + r of the sub-step;
+// with MASK, keys whose offset 16*sg + r exceeds lim (already reduced by 4*(lane/16)) are hidden.
 template <bool MASK>
-__device__ __forceinline__ float lse_fast(const f32x16& acc, float scale2, float mref, float l, int lim) {
+__device__ __forceinline__ float lse_fast(const f32x4 (&a)[2], float scale2, float mref, float l, int lim) {
   const float nm = -mref;
   float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    float x = fmaf(acc[r], scale2, nm);
-    if (MASK) x = (reg_row(r) <= lim) ? x : kNegInf;
-    if (r & 1) s1 += fast_exp2(x); else s0 += fast_exp2(x);
-  }
+  for (int sg = 0; sg < 2; ++sg)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float x = fmaf(a[sg][r], scale2, nm);
+      if (MASK) x = (16 * sg + r <= lim) ? x : kNegInf;
+      if (sg) s1 += fast_exp2(x); else s0 += fast_exp2(x);
+    }
   return l + (s0 + s1);
 }
 
 __device__ __forceinline__ bool lse_in_range(float l) { return (l >= 1.0f) && (l < 1.8446744e19f); }
 
 template <bool MASK>
-__device__ __forceinline__ void lse_renorm(const f32x16& acc, float scale2, float& mref, float& l, int lim) {
+__device__ __forceinline__ void lse_renorm(const f32x4 (&a)[2], float scale2, float& mref, float& l, int lim) {
   const float nm = -mref;
-  float t[16];
+  float t[8];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    float x = fmaf(acc[r], scale2, nm);
-    if (MASK) x = (reg_row(r) <= lim) ? x : kNegInf;
-    t[r] = x;
-  }
+  for (int sg = 0; sg < 2; ++sg)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float x = fmaf(a[sg][r], scale2, nm);
+      if (MASK) x = (16 * sg + r <= lim) ? x : kNegInf;
+      t[sg * 4 + r] = x;
+    }
   float tmax = t[0];
 #pragma unroll
-  for (int r = 1; r < 16; ++r) tmax = fmaxf(tmax, t[r]);
+  for (int i = 1; i < 8; ++i) tmax = fmaxf(tmax, t[i]);
   // Nothing seen yet: the tile maximum becomes the reference (it may be far below zero, so the
   // empty sum must not be scaled: 0 * 2^(+big) is not a number).  Otherwise only ever move up.
   const bool empty = (l == 0.f);
   const float delta = empty ? ((tmax > kNegInf) ? tmax : 0.f) : fmaxf(tmax, 0.f);
   float s = 0.f;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) s += fast_exp2(t[r] - delta);
+  for (int i = 0; i < 8; ++i) s += fast_exp2(t[i] - delta);
   l = empty ? s : l * fast_exp2(-delta) + s;
   mref += delta;
 }
 
 template <bool MASK>
-__device__ __forceinline__ void lse_update(const f32x16& acc, float scale2, float& mref, float& l, int lim) {
-  const float ln = lse_fast<MASK>(acc, scale2, mref, l, lim);
+__device__ __forceinline__ void lse_update(const f32x4 (&a)[2], float scale2, float& mref, float& l, int lim) {
+  const float ln = lse_fast<MASK>(a, scale2, mref, l, lim);
   if (__builtin_amdgcn_ballot_w64(!lse_in_range(ln)) == 0) l = ln;
-  else lse_renorm<MASK>(acc, scale2, mref, l, lim);
+  else lse_renorm<MASK>(a, scale2, mref, l, lim);
 }
 
-// All blocks of a fully visible sub-step; one rarely taken branch at the very end so that the
+// All groups of a fully visible sub-step; one rarely taken branch at the very end so that the
 // arithmetic above it can be scheduled against the MFMAs of the next sub-step.
-template <int NB>
-__device__ __forceinline__ void lse_update_blocks(const f32x16 (&a)[NB], float scale2, float (&mref)[NB],
-                                                  float (&l)[NB]) {
-  float ln[NB];
+template <int NG>
+__device__ __forceinline__ void lse_update_groups(const f32x4 (&a)[NG][2], float scale2, float (&mref)[NG],
+                                                  float (&l)[NG]) {
+  float ln[NG];
   bool ok = true;
 #pragma unroll
-  for (int blk = 0; blk < NB; ++blk) {
-    ln[blk] = lse_fast<false>(a[blk], scale2, mref[blk], l[blk], 0);
-    ok = ok && lse_in_range(ln[blk]);
+  for (int g = 0; g < NG; ++g) {
+    ln[g] = lse_fast<false>(a[g], scale2, mref[g], l[g], 0);
+    ok = ok && lse_in_range(ln[g]);
   }
   if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
 #pragma unroll
-    for (int blk = 0; blk < NB; ++blk) l[blk] = ln[blk];
+    for (int g = 0; g < NG; ++g) l[g] = ln[g];
   } else {
 #pragma unroll
-    for (int blk = 0; blk < NB; ++blk) lse_renorm<false>(a[blk], scale2, mref[blk], l[blk], 0);
+    for (int g = 0; g < NG; ++g) lse_renorm<false>(a[g], scale2, mref[g], l[g], 0);
   }
 }
 
@@ -360,24 +385,26 @@ __device__ __forceinline__ float lse_merge(float a, float b) {
   return hi + fast_log2(1.0f + fast_exp2(lo - hi));
 }
 
+struct NoAux {};
+
 template <int DT, int KS, bool CAUSAL>
 __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   using St = Stager<KS>;
-  constexpr int NB = blocks_per_wave(KS);
+  constexpr int NB = blocks_per_wave(KS), NG = 2 * NB;
   constexpr int kTileRows = tile_rows(KS);
   __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
   int bh, tile, split;
   map_block_split(p, CAUSAL, bh, tile, split);
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lets addresses stay scalar
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, keeps the row views scalar
   const int b = bh / p.H, h = bh - b * p.H;
   const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
   const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
 
-  int q0[NB];  // first query of each of this wave's blocks
-  wave_blocks<NB>(tile, wave, q0);
-  u32x4 qf[NB][KS];
-  load_resident<KS, NB>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
+  int q0[NG];  // first query of each of this wave's groups
+  wave_groups<NB>(tile, wave, q0);
+  u32x4 qf[NG][KS];
+  load_resident<KS, NG>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
 
   // Keys [0, kend) matter to this workgroup.  Chunks [0, t_int) are seen in full by every one of
   // its queries and lie inside [0, N): they take the branch-free pipelined sweep.  The rest (the
@@ -390,14 +417,14 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   const int nchunks = min((kend + kChunk - 1) / kChunk, c_begin + per_split);
   const int t_int = min(nchunks, CAUSAL ? min((tile * kTileRows + p.c + 1) / kChunk, p.N / kChunk) : p.N / kChunk);
 
-  float mref[NB], l[NB];
-  int last[NB];  // last key a lane's query may see, minus the lane's row offset in a block
+  float mref[NG], l[NG];
+  int last[NG];  // last key a lane's query may see, minus the lane's row offset in a group
 #pragma unroll
-  for (int blk = 0; blk < NB; ++blk) {
-    mref[blk] = 0.f;
-    l[blk] = 0.f;
-    const int i = q0[blk] + (lane & 31);
-    last[blk] = (CAUSAL ? min(p.N - 1, i + p.c) : p.N - 1) - 4 * (lane >> 5);
+  for (int g = 0; g < NG; ++g) {
+    mref[g] = 0.f;
+    l[g] = 0.f;
+    const int i = q0[g] + (lane & 15);
+    last[g] = (CAUSAL ? min(p.N - 1, i + p.c) : p.N - 1) - 4 * (lane >> 4);
   }
 
   St st;
@@ -409,10 +436,10 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   stage_store(smem + (c_begin & 1) * St::kBytes);
   stage_load(c_begin + 1);
 
-  pipelined_sweep<DT, KS, NB, false>(
+  pipelined_sweep<DT, KS, NG, false, NoAux>(
       c_begin, t_int, qf, smem, St::kBytes, lane, stage_store, stage_load,
-      [](const char*, int) { return 0.f; },
-      [&](const f32x16(&a)[NB], float) { lse_update_blocks<NB>(a, p.scale2, mref, l); });
+      [](const char*, int) { return NoAux{}; },
+      [&](const f32x4(&a)[NG][2], NoAux) { lse_update_groups<NG>(a, p.scale2, mref, l); });
 
   for (int t = max(t_int, c_begin); t < nchunks; ++t) {
     __syncthreads();  // chunk t published, the other buffer is free
@@ -424,27 +451,30 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
       const int key0 = t * kChunk + sub * 32;
       if (key0 >= p.N) continue;
 #pragma unroll
-      for (int blk = 0; blk < NB; ++blk) {
-        const int qblk = q0[blk];
-        if (CAUSAL && key0 > qblk + 31 + p.c) continue;  // block cannot see this sub-tile
-        f32x16 acc = {0};
+      for (int g = 0; g < NG; ++g) {
+        const int qg = q0[g];
+        if (CAUSAL && key0 > qg + 15 + p.c) continue;  // no query of the group sees this sub-tile
+        f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) acc = mma<DT>(St::frag(lds, sub, ks, lane), qf[blk][ks], acc);
-        const bool need_mask = (key0 + 32 > p.N) || (CAUSAL && key0 + 31 > qblk + p.c);
-        if (need_mask) lse_update<true>(acc, p.scale2, mref[blk], l[blk], last[blk] - key0);
-        else lse_update<false>(acc, p.scale2, mref[blk], l[blk], 0);
+        for (int ks = 0; ks < KS; ++ks) {
+          acc[0] = mma<DT>(St::frag(lds, sub, 0, ks, lane), qf[g][ks], acc[0]);
+          acc[1] = mma<DT>(St::frag(lds, sub, 1, ks, lane), qf[g][ks], acc[1]);
+        }
+        const bool need_mask = (key0 + 32 > p.N) || (CAUSAL && key0 + 31 > qg + p.c);
+        if (need_mask) lse_update<true>(acc, p.scale2, mref[g], l[g], last[g] - key0);
+        else lse_update<false>(acc, p.scale2, mref[g], l[g], 0);
       }
     }
   }
 
 #pragma unroll
-  for (int blk = 0; blk < NB; ++blk) {
-    float v = (l[blk] > 0.f) ? mref[blk] + fast_log2(l[blk]) : kNegInf;
-    const float o = __shfl_xor(v, 32);
-    v = lse_merge(v, o);
-    const int i = q0[blk] + lane;
+  for (int g = 0; g < NG; ++g) {
+    float v = (l[g] > 0.f) ? mref[g] + fast_log2(l[g]) : kNegInf;
+    v = lse_merge(v, __shfl_xor(v, 16));  // the four lane groups hold different keys of the same query
+    v = lse_merge(v, __shfl_xor(v, 32));
+    const int i = q0[g] + lane;
     float* dst = (p.splits > 1) ? p.part + (int64_t)split * p.bh_count * p.M : p.lse;
-    if (lane < 32 && i < p.M) dst[(int64_t)bh * p.M + i] = v;
+    if (lane < 16 && i < p.M) dst[(int64_t)bh * p.M + i] = v;
   }
 }
 
@@ -465,19 +495,27 @@ __global__ __launch_bounds__(256) void lse_combine_kernel(const float* __restric
 // What a column sweep produces.
 constexpr int kModeSum = 0, kModeMax = 1, kModeBoth = 2;
 
-// x = s*scale2 - lse is the base-2 log of the probability.  Sums add 2^x; maxima track x itself and
-// exponentiate once at the end of the sweep (2^x is monotone), so a max-only sweep has no exp.
+// a[sg][r] is the score of key 4*(lane/16) + r of a resident group against the lane's query in
+// streamed group sg, whose lse is lse2[sg].  x = s*scale2 - lse is the base-2 log of the probability.
+// Sums add 2^x; maxima track x itself and exponentiate once at the end of the sweep (2^x is monotone),
+// so a max-only sweep has no exp.  With MASK, register r of group sg is hidden when r > lim + 16*sg.
 template <bool MASK, int MODE>
-__device__ __forceinline__ void col_update(const f32x16& acc, float scale2, float nlse, f32x16& csum,
-                                           f32x16& cmax, int lim) {
+__device__ __forceinline__ void col_update(const f32x4 (&a)[2], float scale2, const float (&lse2)[2], f32x4& csum,
+                                           f32x4& cmax, int lim) {
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    float x = fmaf(acc[r], scale2, nlse);
-    if (MASK) x = (reg_row(r) <= lim) ? x : kNegInf;
-    if (MODE != kModeSum) cmax[r] = fmaxf(cmax[r], x);
-    if (MODE != kModeMax) csum[r] += fast_exp2(x);
-  }
+  for (int sg = 0; sg < 2; ++sg)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      float x = fmaf(a[sg][r], scale2, -lse2[sg]);
+      if (MASK) x = (r <= lim + 16 * sg) ? x : kNegInf;
+      if (MODE != kModeSum) cmax[r] = fmaxf(cmax[r], x);
+      if (MODE != kModeMax) csum[r] += fast_exp2(x);
+    }
 }
+
+struct LsePair {
+  float v[2];
+};
 
 // MODE both keeps two sets of column registers, so a wave then holds one block of keys instead of two.
 __host__ __device__ constexpr int col_blocks_per_wave(int ksteps, int mode) {
@@ -487,34 +525,32 @@ __host__ __device__ constexpr int col_blocks_per_wave(int ksteps, int mode) {
 template <int DT, int KS, bool CAUSAL, int MODE>
 __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p) {
   using St = Stager<KS>;
-  constexpr int NB = col_blocks_per_wave(KS, MODE);
+  constexpr int NB = col_blocks_per_wave(KS, MODE), NG = 2 * NB;
   constexpr int kTileRows = kWaves * 32 * NB;
   constexpr int kStage = St::kBytes + kChunk * 4;     // rows + their lse
-  constexpr int kRed = kWaves * NB * 16 * 64 * 4;     // end-of-sweep transpose buffer
+  constexpr int kRed = kWaves * NG * 4 * 64 * 4;      // end-of-sweep transpose buffer
   constexpr int kSmem = (2 * kStage > kRed) ? 2 * kStage : kRed;
   __shared__ __attribute__((aligned(16))) char smem[kSmem];
   int bh, tile;
   map_block(p, false, bh, tile);
   const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, lets addresses stay scalar
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, keeps the row views scalar
   const int b = bh / p.H, h = bh - b * p.H;
   const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
   const char* kb = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh;
   const float* lse = p.lse + (int64_t)bh * p.M;
 
-  int k0[NB];  // first key of each of this wave's blocks
-  wave_blocks<NB>(tile, wave, k0);
-  u32x4 kf[NB][KS];
-  load_resident<KS, NB>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
+  int k0[NG];  // first key of each of this wave's groups
+  wave_groups<NB>(tile, wave, k0);
+  u32x4 kf[NG][KS];
+  load_resident<KS, NG>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
 
-  f32x16 csum[NB], cmax[NB];  // the set a MODE does not use is never touched and costs no registers
+  f32x4 csum[NG], cmax[NG];  // the set a MODE does not use is never touched and costs no registers
 #pragma unroll
-  for (int blk = 0; blk < NB; ++blk)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      csum[blk][r] = 0.f;
-      cmax[blk][r] = kNegInf;
-    }
+  for (int g = 0; g < NG; ++g) {
+    csum[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    cmax[g] = (f32x4){kNegInf, kNegInf, kNegInf, kNegInf};
+  }
 
   // Query chunks [t0, nchunks) can see keys of this tile.  From chunk t_int on every query sees
   // all of them: those chunks take the branch-free pipelined sweep (rows past M carry lse = +inf
@@ -522,8 +558,8 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
   const int nchunks = (p.M + kChunk - 1) / kChunk;
   const int t0 = CAUSAL ? max(0, tile * kTileRows - p.c) / kChunk : 0;
   const int t_int = CAUSAL ? min(nchunks, max(t0, (tile * kTileRows + kTileRows - 1 - p.c + kChunk - 1) / kChunk)) : 0;
-  // lim = i + c - key0(blk) - 4*(lane/32), with i the lane's query in the current sub-tile
-  const int lim_lane = (lane & 31) + p.c - 4 * (lane >> 5);
+  // lim = i + c - key0(group) - 4*(lane/16), with i the lane's query in group 0 of the current sub-tile
+  const int lim_lane = (lane & 15) + p.c - 4 * (lane >> 4);
 
   // A stage is kChunk query rows plus their lse.  The lse value loaded for chunk t is first
   // touched when the stage is stored, a chunk after its load was issued.
@@ -543,6 +579,10 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
     // +inf for rows past M: they contribute 2^-inf = 0
     reinterpret_cast<float*>(lds + St::kBytes)[tid & (kChunk - 1)] = lse_live ? lse_reg : kPosInf;
   };
+  auto aux_of = [&](const char* lds, int sub) {
+    const float* v = reinterpret_cast<const float*>(lds + St::kBytes) + sub * 32 + (lane & 15);
+    return LsePair{{v[0], v[16]}};
+  };
   stage_load(t0);
   stage_store(smem + (t0 & 1) * kStage);
   stage_load(t0 + 1);
@@ -552,71 +592,71 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
     stage_store(smem + ((t + 1) & 1) * kStage);
     stage_load(t + 2);
     const char* lds = smem + (t & 1) * kStage;
-    const float* lds_lse = reinterpret_cast<const float*>(lds + St::kBytes);
 #pragma unroll
     for (int sub = 0; sub < kChunk / 32; ++sub) {
       const int qs = t * kChunk + sub * 32;  // first query of the sub-tile
       if (qs >= p.M) continue;
-      const float nlse = -lds_lse[sub * 32 + (lane & 31)];
+      const LsePair lq = aux_of(lds, sub);
 #pragma unroll
-      for (int blk = 0; blk < NB; ++blk) {
-        const int kblk = k0[blk];
-        if (kblk >= p.N) continue;
-        if (CAUSAL && kblk > qs + 31 + p.c) continue;  // no query of the sub-tile sees this block
-        f32x16 acc = {0};
+      for (int g = 0; g < NG; ++g) {
+        const int kg = k0[g];
+        if (kg >= p.N) continue;
+        if (CAUSAL && kg > qs + 31 + p.c) continue;  // no query of the sub-tile sees this group
+        f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks) acc = mma<DT>(kf[blk][ks], St::frag(lds, sub, ks, lane), acc);
-        const bool need_mask = CAUSAL && (kblk + 31 > qs + p.c);
-        if (need_mask) col_update<true, MODE>(acc, p.scale2, nlse, csum[blk], cmax[blk], lim_lane + qs - kblk);
-        else col_update<false, MODE>(acc, p.scale2, nlse, csum[blk], cmax[blk], 0);
+        for (int ks = 0; ks < KS; ++ks) {
+          acc[0] = mma<DT>(kf[g][ks], St::frag(lds, sub, 0, ks, lane), acc[0]);
+          acc[1] = mma<DT>(kf[g][ks], St::frag(lds, sub, 1, ks, lane), acc[1]);
+        }
+        const bool need_mask = CAUSAL && (kg + 15 > qs + p.c);
+        if (need_mask) col_update<true, MODE>(acc, p.scale2, lq.v, csum[g], cmax[g], lim_lane + qs - kg);
+        else col_update<false, MODE>(acc, p.scale2, lq.v, csum[g], cmax[g], 0);
       }
     }
   }
 
-  pipelined_sweep<DT, KS, NB, true>(
-      t_int, nchunks, kf, smem, kStage, lane, stage_store, stage_load,
-      [&](const char* lds, int sub) {
-        return reinterpret_cast<const float*>(lds + St::kBytes)[sub * 32 + (lane & 31)];
-      },
-      [&](const f32x16(&a)[NB], float lse_q) {
-        // negated inside the fma, so the LDS read above is first waited for a sub-step later
+  pipelined_sweep<DT, KS, NG, true, LsePair>(
+      t_int, nchunks, kf, smem, kStage, lane, stage_store, stage_load, aux_of,
+      [&](const f32x4(&a)[NG][2], const LsePair& lq) {
+        // the lse values are first touched here, a sub-step after their LDS read was issued
 #pragma unroll
-        for (int blk = 0; blk < NB; ++blk)
-          col_update<false, MODE>(a[blk], p.scale2, -lse_q, csum[blk], cmax[blk], 0);
+        for (int g = 0; g < NG; ++g) col_update<false, MODE>(a[g], p.scale2, lq.v, csum[g], cmax[g], 0);
       });
 
-  // Reduce over the 32 query lanes: transpose through LDS, one output key per lane.
-  float* red = reinterpret_cast<float*>(smem) + wave * (NB * 16 * 64);
-  const int w = lane & 31;
-  const int idx = (lane >> 5) * 16 + (w >> 3) * 4 + (w & 3);
-  const float* src = red + idx * 64 + ((w >> 2) & 1) * 32;
-  const int key = k0[(lane >> 5) < NB ? (lane >> 5) : 0] + w;
-  const bool writer = ((lane >> 5) < NB) && key < p.N;  // lanes 32.. idle when a wave keeps one block
+  // Reduce over the 16 query lanes: transpose through LDS, one output key per lane.
+  float* red = reinterpret_cast<float*>(smem) + wave * (NG * 4 * 64);
+  const int w = lane & 15;                 // key inside its group
+  const int grp = lane >> 4;               // which of the wave's groups this lane writes out
+  const int idx = grp * 4 + (w & 3);
+  const float* src = red + idx * 64 + (w >> 2) * 16;
+  const int key = k0[grp < NG ? grp : 0] + w;
+  const bool active = grp < NG;            // lanes 32.. idle when a wave keeps two groups
+  const bool writer = active && key < p.N;
   if (MODE != kModeMax) {
     __syncthreads();
 #pragma unroll
-    for (int blk = 0; blk < NB; ++blk)
+    for (int g = 0; g < NG; ++g)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) red[(blk * 16 + r) * 64 + lane] = csum[blk][r];
+      for (int r = 0; r < 4; ++r) red[(g * 4 + r) * 64 + lane] = csum[g][r];
     __syncthreads();
-    if ((lane >> 5) < NB) {
+    if (active) {
       float v = 0.f;
-#pragma unroll 8
-      for (int j = 0; j < 32; ++j) v += src[(j + lane) & 31];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) v += src[(j + lane) & 15];
       if (writer) p.out[(int64_t)bh * p.N + key] = v;
     }
   }
   if (MODE != kModeSum) {
     __syncthreads();
 #pragma unroll
-    for (int blk = 0; blk < NB; ++blk)
+    for (int g = 0; g < NG; ++g)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) red[(blk * 16 + r) * 64 + lane] = cmax[blk][r];
+      for (int r = 0; r < 4; ++r) red[(g * 4 + r) * 64 + lane] = cmax[g][r];
     __syncthreads();
-    if ((lane >> 5) < NB) {
+    if (active) {
       float v = kNegInf;
-#pragma unroll 8
-      for (int j = 0; j < 32; ++j) v = fmaxf(v, src[(j + lane) & 31]);
+#pragma unroll
+      for (int j = 0; j < 16; ++j) v = fmaxf(v, src[(j + lane) & 15]);
       float* dst = (MODE == kModeBoth) ? p.out2 : p.out;
       if (writer) dst[(int64_t)bh * p.N + key] = fast_exp2(v);
     }
@@ -753,10 +793,10 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   if (!q || !k || !qs || !ks) return fail(FCR_E_NULL, "null pointer argument");
   if (dtype != FCR_DTYPE_F16 && dtype != FCR_DTYPE_BF16) return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16 or FCR_DTYPE_BF16");
   if (B < 1 || H < 1 || M < 1 || N < 1) return fail(FCR_E_SHAPE, "B, H, M, N must be >= 1");
-  if (D < 8 || D > 16 * kMaxKSteps || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 256]");
+  if (D < 8 || D > 32 * kMaxKSteps || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 256]");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
-  const int trows = by_keys ? kWaves * 32 * col_blocks_per_wave((D + 15) / 16, col_mode) : tile_rows((D + 15) / 16);
+  const int trows = by_keys ? kWaves * 32 * col_blocks_per_wave((D + 31) / 32, col_mode) : tile_rows((D + 31) / 32);
   const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
   if (bh * tiles > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
   if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
@@ -787,7 +827,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
 // workgroup per CU; otherwise the keys of a tile are split so that about two per CU run, each
 // keeping at least four 64-key chunks.
 int row_splits(int B, int H, int M, int N, int D) {
-  const int trows = tile_rows((D + 15) / 16);
+  const int trows = tile_rows((D + 31) / 32);
   const int64_t wgs = (int64_t)B * H * ((M + trows - 1) / trows);
   const int64_t chunks = (N + kChunk - 1) / kChunk;
   if (wgs >= 256 || chunks < 16) return 1;
@@ -834,15 +874,7 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
     case 5: CALL(DT, 5); break;                            \
     case 6: CALL(DT, 6); break;                            \
     case 7: CALL(DT, 7); break;                            \
-    case 8: CALL(DT, 8); break;                            \
-    case 9: CALL(DT, 9); break;                            \
-    case 10: CALL(DT, 10); break;                          \
-    case 11: CALL(DT, 11); break;                          \
-    case 12: CALL(DT, 12); break;                          \
-    case 13: CALL(DT, 13); break;                          \
-    case 14: CALL(DT, 14); break;                          \
-    case 15: CALL(DT, 15); break;                          \
-    default: CALL(DT, 16); break;                          \
+    default: CALL(DT, 8); break;                           \
   }
 
 }  // namespace
@@ -871,7 +903,7 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
   p.splits = row_splits(B, H, M, N, D);
   p.part = lse + (int64_t)B * H * M;  // only touched when splits > 1 (see fcr_lse_bytes)
   p.total *= p.splits;
-  const int ksteps = (D + 15) / 16;
+  const int ksteps = (D + 31) / 32;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal != 0, s)
   if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_LSE) }
@@ -896,7 +928,7 @@ int col_reduce_any(const void* q, const void* k, const float* lse, float* out, f
   p.lse = const_cast<float*>(lse);
   p.out = out;
   p.out2 = out2;
-  const int ksteps = (D + 15) / 16;
+  const int ksteps = (D + 31) / 32;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal != 0, mode, s)
   if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_COL) }
@@ -935,7 +967,7 @@ int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, in
   if (rows < 1 || D < 1) return fail(FCR_E_SHAPE, "rows and D must be >= 1");
   if (terms != 1 && terms != 3) return fail(FCR_E_SHAPE, "terms must be 1 or 3");
   const int dpad = (D + 7) / 8 * 8;
-  if (terms * dpad > 16 * kMaxKSteps) return fail(FCR_E_SHAPE, "terms * D (padded to 8) must be <= 256");
+  if (terms * dpad > 32 * kMaxKSteps) return fail(FCR_E_SHAPE, "terms * D (padded to 8) must be <= 256");
   const int64_t n = rows * dpad;
   if ((n + 255) / 256 > 0x7fffffffll) return fail(FCR_E_SHAPE, "too many elements");
   hipLaunchKernelGGL(pack_f32_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0,
