@@ -35,8 +35,8 @@ HBM_TRAFFIC_BYTES = {"row_lse_kernel": 197.4e6 + 1.05e6, "col_reduce_kernel": 17
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cpu-heads", type=int, default=32,
                     help="heads of the workload the CPU oracle is timed on (0 = skip)")
     ap.add_argument("--copy-calib", action="store_true",

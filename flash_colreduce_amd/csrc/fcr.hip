@@ -311,16 +311,16 @@ __device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&re
 template <bool MASK>
 __device__ __forceinline__ float lse_fast(const f32x4 (&a)[2], float scale2, float mref, float l, int lim) {
   const float nm = -mref;
-  float s0 = 0.f, s1 = 0.f;
+  float ln = l;  // one add per score and nothing else: the groups of a wave give the adder its parallelism
 #pragma unroll
   for (int sg = 0; sg < 2; ++sg)
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       float x = fmaf(a[sg][r], scale2, nm);
       if (MASK) x = (16 * sg + r <= lim) ? x : kNegInf;
-      if (sg) s1 += fast_exp2(x); else s0 += fast_exp2(x);
+      ln += fast_exp2(x);
     }
-  return l + (s0 + s1);
+  return ln;
 }
 
 __device__ __forceinline__ bool lse_in_range(float l) { return (l >= 1.0f) && (l < 1.8446744e19f); }
@@ -364,12 +364,17 @@ template <int NG>
 __device__ __forceinline__ void lse_update_groups(const f32x4 (&a)[NG][2], float scale2, float (&mref)[NG],
                                                   float (&l)[NG]) {
   float ln[NG];
-  bool ok = true;
 #pragma unroll
-  for (int g = 0; g < NG; ++g) {
-    ln[g] = lse_fast<false>(a[g], scale2, mref[g], l[g], 0);
-    ok = ok && lse_in_range(ln[g]);
+  for (int g = 0; g < NG; ++g) ln[g] = lse_fast<false>(a[g], scale2, mref[g], l[g], 0);
+  // one range check for all groups, on the smallest and the largest sum (NaN scores stay NaN on
+  // either path, so they need no test of their own)
+  float lo = ln[0], hi = ln[0];
+#pragma unroll
+  for (int g = 1; g < NG; ++g) {
+    lo = fminf(lo, ln[g]);
+    hi = fmaxf(hi, ln[g]);
   }
+  const bool ok = (lo >= 1.0f) && (hi < 1.8446744e19f);
   if (__builtin_amdgcn_ballot_w64(!ok) == 0) {
 #pragma unroll
     for (int g = 0; g < NG; ++g) l[g] = ln[g];
