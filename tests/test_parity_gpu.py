@@ -341,6 +341,63 @@ def test_topk_on_reduced_columns():
     assert mask[..., 0].all()   # the sink column is always kept
 
 
+def test_random_shapes_against_oracle():
+    """Seeded sweep over shapes, dtypes, masks, scales and layouts that no other test names."""
+    import random
+    rng = random.Random(20240607)
+    for case in range(60):
+        b, h = rng.randint(1, 3), rng.randint(1, 5)
+        m = rng.choice([1, 2, 15, 16, 17, 31, 33, 63, 64, 65, 100, 127, 129, 255, 257, 400, 513, 700])
+        n = rng.choice([1, 3, 16, 17, 32, 63, 65, 128, 130, 255, 256, 257, 300, 511, 640, 1025, 2100])
+        d = rng.choice([8, 16, 24, 32, 40, 64, 72, 96, 100, 128, 136, 160, 192, 256])
+        dtype = rng.choice([torch.float16, torch.bfloat16])
+        causal = rng.random() < 0.5
+        scale = rng.choice([None, None, 0.07, 0.3])
+        q, k = _inputs.randn_pair(b, h, m, n, d, seed=1000 + case, dtype=dtype)
+        if rng.random() < 0.3:  # [B, rows, H, D] storage
+            q = q.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+            k = k.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        reds = rng.sample(REDUCTIONS, rng.randint(1, 3))
+        what = f"case {case}: b{b} h{h} m{m} n{n} d{d} {dtype} causal={causal} scale={scale} {reds}"
+        outs = fca.flash_colreduce_multi(q.cuda(), k.cuda(), reds, is_causal=causal, scale=scale,
+                                         out_dtype=torch.float32)
+        for red, got in zip(reds, outs):
+            check(got, colreduce_ref(q, k, red, causal, scale=scale), red, what)
+
+
+def test_hip_graph_capture_and_replay():
+    """The whole call (torch allocations, both kernels, cast) captured in a graph and replayed with
+    new contents in the static inputs; every replay must equal the eager result for those contents."""
+    b, h, m, n, d = 1, 4, 300, 500, 64
+    qs = torch.zeros(b, h, m, d, device="cuda", dtype=torch.float16)
+    ks = torch.zeros(b, h, n, d, device="cuda", dtype=torch.float16)
+    q0, k0 = _inputs.randn_pair(b, h, m, n, d, seed=77)
+    qs.copy_(q0)
+    ks.copy_(k0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm up outside the capture
+        fca.flash_colreduce_multi(qs, ks, ["sum", "max"], True, out_dtype=torch.float32)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        s_out, m_out = fca.flash_colreduce_multi(qs, ks, ["sum", "max"], True, out_dtype=torch.float32)
+        one = fca.flash_colreduce(qs, ks, "mean", True, out_dtype=torch.float32)
+    for seed in (78, 79, 80):
+        q1, k1 = _inputs.randn_pair(b, h, m, n, d, seed=seed)
+        qs.copy_(q1)
+        ks.copy_(k1)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = (s_out.clone(), m_out.clone(), one.clone())
+        es, em = fca.flash_colreduce_multi(qs, ks, ["sum", "max"], True, out_dtype=torch.float32)
+        e1 = fca.flash_colreduce(qs, ks, "mean", True, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        assert torch.equal(got[0], es) and torch.equal(got[1], em) and torch.equal(got[2], e1), seed
+        check(got[0], colreduce_ref(q1, k1, "sum", True), "sum", f"graph replay seed {seed}")
+
+
 def test_python_errors_on_device():
     q = torch.zeros(1, 2, 4, 8, dtype=torch.float16, device="cuda")
     k = torch.zeros(1, 2, 6, 8, dtype=torch.float16, device="cuda")
