@@ -408,8 +408,6 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
 
   int q0[NG];  // first query of each of this wave's groups
   wave_groups<NB>(tile, wave, q0);
-  u32x4 qf[NG][KS];
-  load_resident<KS, NG>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
 
   // Keys [0, kend) matter to this workgroup.  Chunks [0, t_int) are seen in full by every one of
   // its queries and lie inside [0, N): they take the branch-free pipelined sweep.  The rest (the
@@ -432,12 +430,16 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
     last[g] = (CAUSAL ? min(p.N - 1, i + p.c) : p.N - 1) - 4 * (lane >> 4);
   }
 
+  // The first chunk of the streamed operand is requested before the resident one, so that both are
+  // in flight together and the first LDS stage does not wait for the resident fragments.
   St st;
   st.init(p.k_sr, p.dgran, tid);
-  St::clear(smem, 2 * St::kBytes, p.dgran, tid);
   auto stage_store = [&](char* lds) { st.store(lds); };
   auto stage_load = [&](int t) { st.load(kb, p.k_sr, t * kChunk, p.N); };
   stage_load(c_begin);
+  u32x4 qf[NG][KS];
+  load_resident<KS, NG>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
+  St::clear(smem, 2 * St::kBytes, p.dgran, tid);
   stage_store(smem + (c_begin & 1) * St::kBytes);
   stage_load(c_begin + 1);
 
@@ -547,8 +549,6 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
 
   int k0[NG];  // first key of each of this wave's groups
   wave_groups<NB>(tile, wave, k0);
-  u32x4 kf[NG][KS];
-  load_resident<KS, NG>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
 
   f32x4 csum[NG], cmax[NG];  // the set a MODE does not use is never touched and costs no registers
 #pragma unroll
@@ -572,7 +572,6 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
   float lse_reg;
   bool lse_live;
   st.init(p.q_sr, p.dgran, tid);
-  St::clear(smem, 2 * kStage, p.dgran, tid);
   auto stage_load = [&](int t) {
     st.load(qb, p.q_sr, t * kChunk, p.M);
     const int i = t * kChunk + (tid & (kChunk - 1));  // threads 64.. duplicate threads 0..63
@@ -588,7 +587,12 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
     const float* v = reinterpret_cast<const float*>(lds + St::kBytes) + sub * 32 + (lane & 15);
     return LsePair{{v[0], v[16]}};
   };
+  // The first chunk of the streamed operand is requested before the resident one, so that both are
+  // in flight together and the first LDS stage does not wait for the resident fragments.
   stage_load(t0);
+  u32x4 kf[NG][KS];
+  load_resident<KS, NG>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
+  St::clear(smem, 2 * kStage, p.dgran, tid);
   stage_store(smem + (t0 & 1) * kStage);
   stage_load(t0 + 1);
 
