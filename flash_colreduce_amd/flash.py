@@ -52,7 +52,10 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
     ok = (x.stride(3) == 1 and x.data_ptr() % 16 == 0 and
           all(x.stride(i) % 8 == 0 and x.stride(i) >= 0 for i in (0, 1, 2)) and
           x.stride(2) < (1 << 24))
-    return x if ok else x.contiguous()
+    if ok:
+        return x
+    # a contiguous tensor can still start at a misaligned address: contiguous() would hand it back
+    return x.clone(memory_format=torch.contiguous_format) if x.is_contiguous() else x.contiguous()
 
 
 def _pack_f32(x: torch.Tensor, is_key: bool) -> torch.Tensor:

@@ -207,6 +207,12 @@ def test_strided_inputs(causal):
     k2 = torch.randn(b, h, n, 2 * d, generator=g).half()[..., ::2]
     assert k2.stride(3) == 2
     run_all(q, k2, causal, what="d-stride 2")
+    # contiguous but starting 2 bytes off a 16-byte boundary
+    flat = torch.randn(b * h * n * d + 1, generator=g).half().cuda()
+    k3 = flat[1:].view(b, h, n, d)
+    assert k3.is_contiguous() and k3.data_ptr() % 16 != 0
+    got = fca.flash_colreduce(q.cuda(), k3, "sum", is_causal=causal, out_dtype=torch.float32)
+    check(got, colreduce_ref(q, k3.cpu(), "sum", causal), "sum", "misaligned base")
 
 
 @pytest.mark.parametrize("causal", [False, True])
