@@ -404,6 +404,27 @@ def test_hip_graph_capture_and_replay():
         check(got[0], colreduce_ref(q1, k1, "sum", True), "sum", f"graph replay seed {seed}")
 
 
+def test_launcher_stub_of_the_integration_notes():
+    """The ctypes launcher shown to maintainers (the first python block of section 2 of the integration
+    notes) is executed as written, against the built library, and must reproduce flash_colreduce."""
+    import os
+    import re
+    from flash_colreduce_amd import _lib
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    text = open(os.path.join(root, "INTEGRATION.md")).read()
+    section = text[text.index("## 2."):]
+    code = re.search(r"```python\n(.*?)```", section, flags=re.S).group(1)
+    code = code.replace("/path/to/libfcr.so", _lib.LIB_PATH)
+    scope = {}
+    exec(compile(code, "INTEGRATION.md", "exec"), scope)
+    q, k = _inputs.randn_pair(2, 3, 130, 1000, 64, seed=4)
+    qd, kd = q.cuda(), k.cuda()
+    for red, causal in (("sum", True), ("max", False)):
+        got = scope["_flash_colreduce"](qd, kd, red, causal, 0.125)
+        assert got.dtype == torch.float16 and got.shape == (2, 3, 1000)
+        assert torch.equal(got, fca.flash_colreduce(qd, kd, red, is_causal=causal))
+
+
 def test_python_errors_on_device():
     q = torch.zeros(1, 2, 4, 8, dtype=torch.float16, device="cuda")
     k = torch.zeros(1, 2, 6, 8, dtype=torch.float16, device="cuda")
