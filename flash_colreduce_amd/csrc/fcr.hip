@@ -61,6 +61,7 @@ struct Params {
   float scale2;      // scale * log2(e)
   int tiles;         // resident tiles per (b,h)
   int bh_count;      // B * H
+  int group;         // (b,h) pairs whose workgroups are launched together (see map_block)
   int total;         // tiles * B * H workgroups
 };
 
@@ -81,25 +82,36 @@ __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c) {
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ __forceinline__ float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
-// Work order.  Workgroup v takes (b,h) = v % BH and the tile of rank v / BH, tiles ranked by the
-// length of their sweep, longest first: with more workgroups than the chip holds at once, the
-// short ones fill in behind the long ones and the causal triangle finishes level.  Workgroups are
-// dealt to the 8 XCDs round-robin by v, so when BH is a multiple of 8 every (b,h) stays on XCD
-// (b,h) % 8 and its streamed operand is shared through that XCD's L2.
-__device__ __forceinline__ void map_block(const Params& p, bool longest_is_last_tile, int& bh, int& tile) {
+// Work order.  The (b,h) pairs are taken in groups of `group`; inside a group workgroup w takes
+// (b,h) = first + w % g and the tile of rank w / g, tiles ranked by the length of their sweep,
+// longest first: with more workgroups than the chip holds at once, the short ones fill in behind
+// the long ones and the causal triangle finishes level.  A group is sized to about what the chip
+// holds at once, so all tiles of a (b,h) run at the same time and its streamed operand comes from
+// HBM once.  Workgroups are dealt to the 8 XCDs round-robin by v, so with group a multiple of 8
+// every (b,h) stays on XCD (b,h) % 8 and that operand is shared through the XCD's L2.
+__device__ __forceinline__ void map_group(const Params& p, int per_bh, int& bh, int& r) {
   const int v = (int)blockIdx.x;
-  const int rank = v / p.bh_count;
-  bh = v - rank * p.bh_count;
+  const int per = p.group * per_bh;
+  const int chunk = v / per;
+  const int first = chunk * p.group;
+  const int g = min(p.group, p.bh_count - first);
+  const int w = v - chunk * per;
+  r = w / g;
+  bh = first + (w - r * g);
+}
+
+__device__ __forceinline__ void map_block(const Params& p, bool longest_is_last_tile, int& bh, int& tile) {
+  int rank;
+  map_group(p, p.tiles, bh, rank);
   tile = longest_is_last_tile ? p.tiles - 1 - rank : rank;
 }
 
 // Row kernel with the keys of a tile split over several workgroups (few query rows, many keys):
-// workgroup v takes (b,h) = v % BH, then the key range, then the tile.
+// inside a group the order is (b,h), then the key range, then the tile.
 __device__ __forceinline__ void map_block_split(const Params& p, bool longest_is_last_tile, int& bh, int& tile,
                                                 int& split) {
-  const int v = (int)blockIdx.x;
-  const int r = v / p.bh_count;
-  bh = v - r * p.bh_count;
+  int r;
+  map_group(p, p.tiles * p.splits, bh, r);
   const int rank = r / p.splits;
   split = r - rank * p.splits;
   tile = longest_is_last_tile ? p.tiles - 1 - rank : rank;
@@ -797,6 +809,18 @@ int check_strides(const void* ptr, const int64_t s[4], const char* name) {
   return 0;
 }
 
+// (b,h) pairs per launch group, a multiple of 8.  Without a mask all sweeps of a launch are equally
+// long and about one workgroup per CU (256) keeps the tiles of a (b,h) together in time.  With the
+// causal mask the longest-first order needs room to level the triangle: about 1024 workgroups and
+// never fewer than 32 pairs (measured: smaller groups lose up to 8 % on 32 heads of 8192 rows,
+// larger ones up to 11 % on 1024 heads of 2048 rows, whose operands then come from HBM per tile).
+int head_group(int64_t bh, int64_t per_bh, bool causal) {
+  int64_t g = ((causal ? 1024 : 256) / per_bh) & ~7ll;
+  const int64_t least = causal ? 32 : 8;
+  if (g < least) g = least;
+  return (int)(g < bh ? g : bh);
+}
+
 int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H, int M, int N, int D,
                 const int64_t qs[4], const int64_t ks[4], float scale, bool by_keys, int col_mode = kModeSum) {
   if (!q || !k || !qs || !ks) return fail(FCR_E_NULL, "null pointer argument");
@@ -912,6 +936,7 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
   p.splits = row_splits(B, H, M, N, D);
   p.part = lse + (int64_t)B * H * M;  // only touched when splits > 1 (see fcr_lse_bytes)
   p.total *= p.splits;
+  p.group = head_group(p.bh_count, (int64_t)p.tiles * p.splits, causal != 0);
   const int ksteps = (D + 31) / 32;
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal != 0, s)
@@ -934,6 +959,7 @@ int col_reduce_any(const void* q, const void* k, const float* lse, float* out, f
   if (!lse || !out || (mode == kModeBoth && !out2)) return fail(FCR_E_NULL, "null pointer argument");
   int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true, mode);
   if (rc) return rc;
+  p.group = head_group(p.bh_count, p.tiles, causal != 0);
   p.lse = const_cast<float*>(lse);
   p.out = out;
   p.out2 = out2;

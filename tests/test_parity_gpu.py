@@ -186,6 +186,20 @@ def test_few_queries_many_keys(b, h, m, n, d, causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("b,h,m,n,d", [
+    (103, 10, 32, 40, 8),      # one tile per (b,h): 1030 pairs, more than one launch group either way
+    (5, 68, 700, 520, 16),     # three row tiles, 340 pairs: last group is partial
+    (5, 8, 64, 4096, 32),      # split keys, 40 pairs in groups of 16 without the mask
+    (3, 23, 520, 300, 8),      # 69 pairs, not a multiple of 8
+])
+def test_many_heads_in_launch_groups(b, h, m, n, d, causal):
+    """(b,h) pairs are launched in groups; cover more pairs than one group holds, partial last groups
+    and pair counts that are not multiples of 8, for both kernels and the split-key row sweep."""
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=b * h + m)
+    run_all(q, k, causal, what=f"groups b{b} h{h} m{m} n{n} d{d}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
 def test_explicit_and_negative_scale(causal):
     q, k = _inputs.randn_pair(1, 4, 200, 333, 64, seed=21)
     for scale in (0.05, 1.0 / 3.0, -0.125, 0.0):
