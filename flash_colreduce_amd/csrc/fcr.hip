@@ -39,7 +39,22 @@ constexpr int kThreads = kWaves * 64;
 // two 32-row blocks (four groups) while their fragments fit the register file next to the
 // accumulators (D <= 128: 4 k-steps), one block for larger D.  A workgroup keeps 4 * 32 * blocks rows.
 __host__ __device__ constexpr int blocks_per_wave(int ksteps) { return ksteps <= 4 ? 2 : 1; }
-__host__ __device__ constexpr int tile_rows(int ksteps) { return kWaves * 32 * blocks_per_wave(ksteps); }
+// The row kernel has both forms for D <= 128 and the host picks per problem.  Waves whose rows are all
+// padding do no arithmetic, so a launch costs (rows in waves with at least one query) x (cost per
+// row); one block per wave costs about 3 % per k-step more per row (every streamed fragment feeds
+// half as many MFMAs) but rounds M up to 32 instead of 64 rows per wave: it wins for M <= 128 and
+// for a few ragged M above that.
+inline int64_t rows_swept(int M, int nb) {
+  const int trows = kWaves * 32 * nb;
+  const int rem = M % trows;
+  const int waves = rem ? (rem + 31) / 32 : 0;   // blocks of the last tile that hold queries
+  return (int64_t)(M / trows) * trows + (waves < kWaves ? waves : kWaves) * 32 * nb;
+}
+inline int row_blocks_per_wave(int ksteps, int M) {
+  if (ksteps > 4) return 1;
+  return rows_swept(M, 1) * (100 + 3 * ksteps) < rows_swept(M, 2) * 100 ? 1 : 2;
+}
+inline int row_tile_rows(int ksteps, int M) { return kWaves * 32 * row_blocks_per_wave(ksteps, M); }
 constexpr int kMaxKSteps = 8;                 // D <= 256
 constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row sub-steps)
 constexpr float kNegInf = -__builtin_inff();
@@ -265,6 +280,22 @@ __device__ __forceinline__ void mma_groups(f32x4 (&n)[NG][2], u32x4 (&f)[2][KS],
 // aux_of(lds, sub) reads what the consumer needs per sub-step besides the scores (the column
 // kernel: lse of the lane's queries); it travels with the fragments so that it too is read before
 // the barrier that lets other waves overwrite the buffer.
+// staging_sweep below is the same sequence of barriers, LDS stores and global loads without the
+// arithmetic, for a wave whose resident rows are all padding.
+template <class StoreF, class LoadF>
+__device__ __forceinline__ void staging_sweep(int ta, int tb, char* smem, int stage_bytes, StoreF&& stage_store,
+                                              LoadF&& stage_load) {
+  if (ta >= tb) return;
+  __syncthreads();
+  stage_store(smem + ((ta + 1) & 1) * stage_bytes);
+  stage_load(ta + 2);
+  for (int t = ta; t + 1 < tb; ++t) {
+    __syncthreads();
+    stage_store(smem + (t & 1) * stage_bytes);
+    stage_load(t + 3);
+  }
+}
+
 template <int DT, int KS, int NG, bool RESIDENT_IS_KEYS, class Aux, class StoreF, class LoadF, class AuxF,
           class ConsumeF>
 __device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[NG][KS], char* smem,
@@ -404,11 +435,11 @@ __device__ __forceinline__ float lse_merge(float a, float b) {
 
 struct NoAux {};
 
-template <int DT, int KS, bool CAUSAL>
+template <int DT, int KS, bool CAUSAL, int NB>
 __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   using St = Stager<KS>;
-  constexpr int NB = blocks_per_wave(KS), NG = 2 * NB;
-  constexpr int kTileRows = tile_rows(KS);
+  constexpr int NG = 2 * NB;
+  constexpr int kTileRows = kWaves * 32 * NB;
   __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
   int bh, tile, split;
   map_block_split(p, CAUSAL, bh, tile, split);
@@ -454,6 +485,17 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   St::clear(smem, 2 * St::kBytes, p.dgran, tid);
   stage_store(smem + (c_begin & 1) * St::kBytes);
   stage_load(c_begin + 1);
+
+  // A wave whose rows all lie past M (a ragged last tile, fewer than 128 queries) only helps staging.
+  if (q0[0] >= p.M) {
+    staging_sweep(c_begin, t_int, smem, St::kBytes, stage_store, stage_load);
+    for (int t = max(t_int, c_begin); t < nchunks; ++t) {
+      __syncthreads();
+      stage_store(smem + ((t + 1) & 1) * St::kBytes);
+      stage_load(t + 2);
+    }
+    return;
+  }
 
   pipelined_sweep<DT, KS, NG, false, NoAux>(
       c_begin, t_int, qf, smem, St::kBytes, lane, stage_store, stage_load,
@@ -829,7 +871,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   if (D < 8 || D > 32 * kMaxKSteps || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 256]");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
-  const int trows = by_keys ? kWaves * 32 * col_blocks_per_wave((D + 31) / 32, col_mode) : tile_rows((D + 31) / 32);
+  const int trows = by_keys ? kWaves * 32 * col_blocks_per_wave((D + 31) / 32, col_mode) : row_tile_rows((D + 31) / 32, M);
   const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
   if (bh * tiles > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
   if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
@@ -860,7 +902,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
 // workgroup per CU; otherwise the keys of a tile are split so that about two per CU run, each
 // keeping at least four 64-key chunks.
 int row_splits(int B, int H, int M, int N, int D) {
-  const int trows = tile_rows((D + 31) / 32);
+  const int trows = row_tile_rows((D + 31) / 32, M);
   const int64_t wgs = (int64_t)B * H * ((M + trows - 1) / trows);
   const int64_t chunks = (N + kChunk - 1) / kChunk;
   if (wgs >= 256 || chunks < 16) return 1;
@@ -877,11 +919,19 @@ int launched(const char* what) {
   return (int)e;
 }
 
+template <int DT, int KS, int NB>
+void launch_lse_blocks(const Params& p, bool causal, hipStream_t s) {
+  const dim3 grid(p.total), block(kThreads);
+  if (causal) hipLaunchKernelGGL((row_lse_kernel<DT, KS, true, NB>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((row_lse_kernel<DT, KS, false, NB>), grid, block, 0, s, p);
+}
+
 template <int DT, int KS>
 void launch_lse(const Params& p, bool causal, hipStream_t s) {
-  const dim3 grid(p.total), block(kThreads);
-  if (causal) hipLaunchKernelGGL((row_lse_kernel<DT, KS, true>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((row_lse_kernel<DT, KS, false>), grid, block, 0, s, p);
+  if constexpr (KS <= 4) {
+    if (row_blocks_per_wave(KS, p.M) == 2) return launch_lse_blocks<DT, KS, 2>(p, causal, s);
+  }
+  launch_lse_blocks<DT, KS, 1>(p, causal, s);
 }
 
 template <int DT, int KS, int MODE>

@@ -199,6 +199,34 @@ def test_many_heads_in_launch_groups(b, h, m, n, d, causal):
     run_all(q, k, causal, what=f"groups b{b} h{h} m{m} n{n} d{d}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n,d", [
+    (1, 1, 8), (1, 4100, 128), (16, 64, 64), (17, 65, 72), (63, 200, 128), (64, 1100, 128), (64, 10, 32),
+    (33, 4097, 96), (64, 6000, 128), (8, 2048, 16), (64, 129, 136),
+])
+def test_at_most_64_queries(m, n, d, causal, dtype):
+    """Few query rows against few or many keys: the row sweep keeps one 32-row block per wave and the
+    waves without any query only help staging; the causal diagonal is the last M keys.  Also the fused
+    sum+max form."""
+    q, k = _inputs.randn_pair(2, 5, m, n, d, seed=m + 3 * n + d, dtype=dtype)
+    run_all(q, k, causal, what=f"small m{m} n{n} d{d} {dtype}")
+    got = fca.flash_colreduce_multi(q.cuda(), k.cuda(), ("sum", "max"), is_causal=causal, out_dtype=torch.float32)
+    check(got[0], colreduce_ref(q, k, "sum", causal), "sum", f"small fused m{m} n{n} d{d}")
+    check(got[1], colreduce_ref(q, k, "max", causal), "max", f"small fused m{m} n{n} d{d}")
+
+
+@pytest.mark.parametrize("m", [100, 128, 300, 384, 600])
+def test_row_sweep_block_choice(m):
+    """Query counts for which the row sweep keeps one 32-row block per wave (M <= 128 and ragged M
+    such as 300, 384, 600) next to ones that keep two; the last tile has waves without any query."""
+    q, k = _inputs.randn_pair(1, 6, m, 1500, 128, seed=m)
+    for causal in (False, True):
+        got = fca.row_lse2(q.cuda(), k.cuda(), is_causal=causal).double().cpu()
+        torch.testing.assert_close(got, row_lse2_ref(q, k, causal), rtol=0, atol=3e-4)
+        run_all(q, k, causal, what=f"row blocks m{m}", reductions=("sum",))
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_explicit_and_negative_scale(causal):
     q, k = _inputs.randn_pair(1, 4, 200, 333, 64, seed=21)
