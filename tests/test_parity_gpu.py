@@ -227,6 +227,22 @@ def test_row_sweep_block_choice(m):
         run_all(q, k, causal, what=f"row blocks m{m}", reductions=("sum",))
 
 
+def test_key_operand_beyond_4_gib():
+    """One head whose keys take more than 4 GiB: row offsets inside an operand exceed 32 bits and the
+    buffer views are clamped; the last columns lie past that mark.  Relative check only (the sums are
+    far below the absolute tolerance)."""
+    n, d = (1 << 24) + 77, 128
+    g = torch.Generator(device="cuda").manual_seed(3)
+    k = torch.randn(1, 1, n, d, device="cuda", dtype=torch.float16, generator=g)
+    q = torch.randn(1, 1, 4, d, device="cuda", dtype=torch.float16, generator=g)
+    qc, kc = q.cpu(), k.cpu()
+    for causal in (False, True):
+        got_s, got_m = fca.flash_colreduce_multi(q, k, ("sum", "max"), is_causal=causal, out_dtype=torch.float32)
+        for got, red in ((got_s, "sum"), (got_m, "max")):
+            want = colreduce_ref(qc, kc, red, causal, chunk_rows=16)
+            torch.testing.assert_close(got.cpu(), want, rtol=2e-3, atol=0, msg=lambda m: f"{red} causal={causal}: {m}")
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_explicit_and_negative_scale(causal):
     q, k = _inputs.randn_pair(1, 4, 200, 333, 64, seed=21)
