@@ -10,8 +10,9 @@
 // The 16x16x32 shape is used because on this chip it sustains about 14 % more flops per watt than
 // 32x32x16 on random operands, and these kernels run against the package power limit.
 //
-//   row_lse_kernel    a workgroup keeps 256 query rows in registers (64 per wave) and streams
-//                     key tiles through LDS; writes lse2[bh, i] = log2 sum_j 2^(s_ij).
+//   row_lse_kernel    a workgroup keeps 256 query rows in registers (64 per wave; 128 and 32 for
+//                     few or ragged M and for D > 128) and streams key tiles through LDS; writes
+//                     lse2[bh, i] = log2 sum_j 2^(s_ij).
 //   col_reduce_kernel a workgroup keeps 256 key rows in registers and streams query tiles (and
 //                     their lse2) through LDS; writes out[bh, j] = sum_i or max_i 2^(s_ij-lse2_i).
 // where s_ij = scale * log2(e) * <q_i, k_j>.  Nothing of size M*N is written anywhere and there
@@ -184,8 +185,10 @@ __device__ __forceinline__ void load_resident(u32x4 (&f)[NG][KS], const char* ba
 }
 
 // Global -> registers -> LDS staging of kChunk rows of the streamed operand.
-// LDS rows are padded by 16 bytes so that the 16-byte fragment reads of 16 consecutive rows
-// fall into distinct banks.  A thread moves the same granules (row r, 16-byte column cg) of
+// LDS rows are padded by 32 bytes: a 16-byte fragment read is served in passes of lanes {0-7, 16-23},
+// {8-15, 24-31}, .. (eight consecutive rows at two neighbouring 16-byte columns), and with a pitch of
+// 8 banks modulo 64 these fall into distinct banks (SQ_LDS_BANK_CONFLICT = 0; with 16 bytes of padding
+// every read took two passes).  A thread moves the same granules (row r, 16-byte column cg) of
 // every chunk, so its source offset inside a chunk and its LDS offset are computed once.
 // Granule columns at or past D/8 (the zero padding up to the MFMA k-step) are never written
 // (their threads store to a dummy slot): the buffers are cleared once and those columns stay zero.
@@ -193,7 +196,7 @@ __device__ __forceinline__ void load_resident(u32x4 (&f)[NG][KS], const char* ba
 template <int KS>
 struct Stager {
   static constexpr int kGran = 4 * KS;             // 16-byte granules per (zero padded) row
-  static constexpr int kRowBytes = KS * 64 + 16;   // LDS row pitch
+  static constexpr int kRowBytes = KS * 64 + 32;   // LDS row pitch
   static constexpr int kTotal = kChunk * kGran;
   static constexpr int kPer = (kTotal + kThreads - 1) / kThreads;
   static constexpr int kDummy = kChunk * kRowBytes;  // 16 bytes nobody reads
