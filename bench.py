@@ -29,7 +29,7 @@ PEAK_FP16_DENSE_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/CU/clk, MI355X p
 # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # scaled by the same counters on a 256 MiB device copy (FETCH unit 2 KiB, WRITE unit 1 KiB);
 # the summary of those runs is profiles/headline_causal_8192_fp16.md.
-HBM_TRAFFIC_BYTES = {"row_lse_kernel": 198.0e6 + 1.05e6, "col_reduce_kernel": 185.1e6 + 1.05e6}
+HBM_TRAFFIC_BYTES = {"row_lse_kernel": 198.1e6 + 1.05e6, "col_reduce_kernel": 186.0e6 + 1.05e6}
 
 
 def main():
