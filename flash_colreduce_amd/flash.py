@@ -6,6 +6,7 @@ a C ABI (include/fcr.h); torch is used for device memory and the current stream 
 """
 from __future__ import annotations
 
+import functools
 import math
 from typing import Optional
 
@@ -127,6 +128,13 @@ def _launch(query, key, kinds, is_causal, scale):
     return outs, lse[: b * h * m]
 
 
+@functools.lru_cache(maxsize=8)
+def _countdown(count: int, device: torch.device) -> torch.Tensor:
+    """count, count-1, .., 1: the causal mean divisor from the offset on (flash.py:381-382), kept
+    between calls because building it costs more host time than a small problem's kernels."""
+    return torch.arange(count, 0, -1, device=device)
+
+
 def _finish(acc, reduction, query, m, n, is_causal, res_dtype, shared=False):
     """Cast of the fp32 accumulation and the mean epilogue, as flash.py:308 and 377-385.
 
@@ -138,7 +146,7 @@ def _finish(acc, reduction, query, m, n, is_causal, res_dtype, shared=False):
         if is_causal:
             c = max(n - m, 0)
             scores[..., :c] /= m
-            scores[..., c:] /= torch.arange(n - c, 0, -1, device=query.device)
+            scores[..., c:] /= _countdown(n - c, query.device)
         else:
             scores /= m
     return scores
