@@ -161,8 +161,12 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_view(const char* base, in
                                            (int)(uint32_t)bytes, 0x00020000);
 }
 
+// AUX is the cache policy of the load: 0 = default, kLoadOnce = non-temporal, for bytes that no
+// workgroup of the launch will ask for again.
+constexpr int kLoadOnce = 2;
+template <int AUX = 0>
 __device__ __forceinline__ u32x4 view_load16(__amdgpu_buffer_rsrc_t v, uint32_t byte_off) {
-  return __builtin_amdgcn_raw_buffer_load_b128(v, (int)byte_off, 0, 0);
+  return __builtin_amdgcn_raw_buffer_load_b128(v, (int)byte_off, 0, AUX);
 }
 
 // The operand a wave keeps for the whole sweep: NG groups of 16 rows starting at rows[g], as MFMA
@@ -224,10 +228,11 @@ struct Stager {
     }
   }
   // Rows [row0, row0 + kChunk) of an operand of nrows rows starting at base.  No branches.
+  template <int AUX = 0>
   __device__ __forceinline__ void load(const char* base, int64_t row_bytes, int row0, int nrows) {
     const __amdgpu_buffer_rsrc_t view = rows_view(base, row_bytes, row0, nrows);
 #pragma unroll
-    for (int i = 0; i < kPer; ++i) regs[i] = view_load16(view, goff[i]);
+    for (int i = 0; i < kPer; ++i) regs[i] = view_load16<AUX>(view, goff[i]);
   }
   __device__ __forceinline__ void store(char* lds) const {
 #pragma unroll
@@ -438,7 +443,11 @@ __device__ __forceinline__ float lse_merge(float a, float b) {
 
 struct NoAux {};
 
-template <int DT, int KS, bool CAUSAL, int NB>
+// STREAM_ONCE: the launch has one row tile per (b,h), so every key is read by exactly one workgroup,
+// and so many keys that none of them survives in a cache until the column kernel: they are loaded
+// non-temporally (7.0 instead of 6.2 TB/s on 34 GB of keys).  With several row tiles, or few keys, the
+// default policy is the faster one.
+template <int DT, int KS, bool CAUSAL, int NB, bool STREAM_ONCE>
 __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   using St = Stager<KS>;
   constexpr int NG = 2 * NB;
@@ -481,7 +490,7 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   St st;
   st.init(p.k_sr, p.dgran, tid);
   auto stage_store = [&](char* lds) { st.store(lds); };
-  auto stage_load = [&](int t) { st.load(kb, p.k_sr, t * kChunk, p.N); };
+  auto stage_load = [&](int t) { st.template load<(STREAM_ONCE ? kLoadOnce : 0)>(kb, p.k_sr, t * kChunk, p.N); };
   stage_load(c_begin);
   u32x4 qf[NG][KS];
   load_resident<KS, NG>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
@@ -922,19 +931,22 @@ int launched(const char* what) {
   return (int)e;
 }
 
-template <int DT, int KS, int NB>
+template <int DT, int KS, int NB, bool ONCE>
 void launch_lse_blocks(const Params& p, bool causal, hipStream_t s) {
   const dim3 grid(p.total), block(kThreads);
-  if (causal) hipLaunchKernelGGL((row_lse_kernel<DT, KS, true, NB>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((row_lse_kernel<DT, KS, false, NB>), grid, block, 0, s, p);
+  if (causal) hipLaunchKernelGGL((row_lse_kernel<DT, KS, true, NB, ONCE>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((row_lse_kernel<DT, KS, false, NB, ONCE>), grid, block, 0, s, p);
 }
 
 template <int DT, int KS>
 void launch_lse(const Params& p, bool causal, hipStream_t s) {
   if constexpr (KS <= 4) {
-    if (row_blocks_per_wave(KS, p.M) == 2) return launch_lse_blocks<DT, KS, 2>(p, causal, s);
+    if (row_blocks_per_wave(KS, p.M) == 2) return launch_lse_blocks<DT, KS, 2, false>(p, causal, s);
   }
-  launch_lse_blocks<DT, KS, 1>(p, causal, s);
+  // one row tile per (b,h) and at least 1 GiB of keys: stream them past the caches
+  const int64_t key_bytes = (int64_t)p.bh_count * p.N * p.dgran * 16;
+  if (p.tiles == 1 && key_bytes >= (1ll << 30)) return launch_lse_blocks<DT, KS, 1, true>(p, causal, s);
+  launch_lse_blocks<DT, KS, 1, false>(p, causal, s);
 }
 
 template <int DT, int KS, int MODE>
