@@ -216,6 +216,26 @@ def test_at_most_64_queries(m, n, d, causal, dtype):
     check(got[1], colreduce_ref(q, k, "max", causal), "max", f"small fused m{m} n{n} d{d}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("b,h,m,n,d", [
+    (4, 16, 64, 4100, 128),    # 64 pairs x 4 key ranges
+    (1, 130, 33, 1030, 64),    # one range per pair, a ragged last chunk, padded query groups
+    (2, 40, 1, 2048, 16),      # a single query
+    (3, 50, 64, 1100, 72),     # D not a multiple of 32
+    (1, 8, 17, 40000, 32),     # many ranges per pair
+])
+def test_few_queries_with_streamed_keys(b, h, m, n, d, causal, dtype):
+    """At most 64 queries, D <= 128 and enough (b,h) pairs x keys to fill the chip: the column
+    sweep with the queries resident in every wave and the keys streamed in ranges; sum, mean, max and
+    the fused sum+max form.  With the mask the diagonal is the last M keys."""
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=b * h + m + n, dtype=dtype)
+    run_all(q, k, causal, what=f"streamed keys b{b} h{h} m{m} n{n} d{d} {dtype}")
+    got = fca.flash_colreduce_multi(q.cuda(), k.cuda(), ("sum", "max"), is_causal=causal, out_dtype=torch.float32)
+    check(got[0], colreduce_ref(q, k, "sum", causal), "sum", "streamed keys fused")
+    check(got[1], colreduce_ref(q, k, "max", causal), "max", "streamed keys fused")
+
+
 @pytest.mark.parametrize("m", [100, 128, 300, 384, 600])
 def test_row_sweep_block_choice(m):
     """Query counts for which the row sweep keeps one 32-row block per wave (M <= 128 and ragged M
