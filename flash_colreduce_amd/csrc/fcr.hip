@@ -126,13 +126,15 @@ __device__ __forceinline__ void map_block(const Params& p, bool longest_is_last_
 }
 
 // Row kernel with the keys of a tile split over several workgroups (few query rows, many keys):
-// inside a group the order is (b,h), then the key range, then the tile.
+// inside a group the order is (b,h), then the tile, then the key range: the tiles that stream the
+// same keys start next to each other on the same XCD and share them through its L2.
 __device__ __forceinline__ void map_block_split(const Params& p, bool longest_is_last_tile, int& bh, int& tile,
                                                 int& split) {
   int r;
   map_group(p, p.tiles * p.splits, bh, r);
-  const int rank = r / p.splits;
-  split = r - rank * p.splits;
+  const int back = r / p.tiles;   // the last key range first: with the mask it holds the diagonal, the slow part
+  const int rank = r - back * p.tiles;
+  split = p.splits - 1 - back;
   tile = longest_is_last_tile ? p.tiles - 1 - rank : rank;
 }
 
