@@ -15,7 +15,7 @@
 //                     lse2[bh, i] = log2 sum_j 2^(s_ij).
 //   col_reduce_kernel a workgroup keeps 256 key rows in registers and streams query tiles (and
 //                     their lse2) through LDS; writes out[bh, j] = sum_i or max_i 2^(s_ij-lse2_i).
-//   col_small_kernel  the same result for at most 64 query rows against many keys: queries resident
+//   col_small_kernel  the same result for at most 128 query rows against many keys: queries resident
 //                     in every wave, keys streamed (HBM bound).
 // where s_ij = scale * log2(e) * <q_i, k_j>.  Nothing of size M*N is written anywhere and there
 // are no atomics: one workgroup owns its output rows / columns.
@@ -744,8 +744,8 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
 }
 
 // ---------------------------------------------------------------------------------------------
-// Column sweep for at most 64 query rows against many keys, where the sweep is bound by reading K.
-// The roles are swapped: every wave keeps ALL queries resident (four groups of 16) and the keys
+// Column sweep for at most 128 query rows against many keys, where the sweep is bound by reading K.
+// The roles are swapped: every wave keeps ALL queries resident (NG = 4 or 8 groups of 16) and the keys
 // stream through LDS in chunks of 64, fully coalesced and two chunks ahead.  Wave w takes keys
 // [16w, 16w+16) of each chunk with S = Q * K^T, so a lane holds one key (lane & 15) against the
 // queries 16g + 4*(lane/16) + r: the column reduction is an in-register sum over g and r plus two
@@ -754,12 +754,11 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
 // one workgroup; p.stream_once makes those loads non-temporal (set when K is too large to stay cached).
 // The general kernel reads the same keys as MFMA fragments, 64 bytes per row and instruction, and
 // reaches 4.9 TB/s where this one reaches 6 (measured on 34 GB of keys).
-constexpr int kSmallRows = 64;
+constexpr int kSmallRows = 128;
 
-template <int DT, int KS, bool CAUSAL, int MODE>
-__global__ __launch_bounds__(kThreads, 3) void col_small_kernel(const Params p) {
+template <int DT, int KS, bool CAUSAL, int MODE, int NG>
+__global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(const Params p) {
   using St = Stager<KS>;
-  constexpr int NG = kSmallRows / 16;
   __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
   int bh, split;
   map_group(p, p.splits, bh, split);
@@ -826,29 +825,33 @@ __global__ __launch_bounds__(kThreads, 3) void col_small_kernel(const Params p) 
     store(r, smem + ((t + 1) & 1) * St::kBytes);
     load(r, t + 3);
     const char* lds = smem + (t & 1) * St::kBytes;
-    f32x4 acc[NG];
-#pragma unroll
-    for (int g = 0; g < NG; ++g) acc[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 kfrag = St::frag(lds, wave >> 1, wave & 1, ks, lane);
-#pragma unroll
-      for (int g = 0; g < NG; ++g) acc[g] = mma<DT>(qf[g][ks], kfrag, acc[g]);
-    }
     const int key = t * kChunk + 16 * wave + (lane & 15);
     // query i sees the key iff key <= i + c; chunks that end at or before key c need no mask
     const bool need_mask = CAUSAL && (t * kChunk + kChunk - 1 > p.c);
     const int first = key - p.c - qrow;  // register (g, r) is visible iff 16g + r >= first
     float vsum = 0.f, vmax = kNegInf;
+    // four query groups at a time, so that at most four accumulators are live
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
+    for (int gb = 0; gb < NG; gb += 4) {
+      f32x4 acc[4];
 #pragma unroll
-      for (int r2 = 0; r2 < 4; ++r2) {
-        float x = fmaf(acc[g][r2], p.scale2, nlse[g][r2]);
-        if (need_mask) x = (16 * g + r2 >= first) ? x : kNegInf;
-        if (MODE != kModeSum) vmax = fmaxf(vmax, x);
-        if (MODE != kModeMax) vsum += fast_exp2(x);
+      for (int g = 0; g < 4; ++g) acc[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4 kfrag = St::frag(lds, wave >> 1, wave & 1, ks, lane);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) acc[g] = mma<DT>(qf[gb + g][ks], kfrag, acc[g]);
       }
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int r2 = 0; r2 < 4; ++r2) {
+          float x = fmaf(acc[g][r2], p.scale2, nlse[gb + g][r2]);
+          if (need_mask) x = (16 * (gb + g) + r2 >= first) ? x : kNegInf;
+          if (MODE != kModeSum) vmax = fmaxf(vmax, x);
+          if (MODE != kModeMax) vsum += fast_exp2(x);
+        }
+    }
     // the four lane groups hold different queries of the same key
     if (MODE != kModeMax) {
       vsum += __shfl_xor(vsum, 16);
@@ -1086,11 +1089,17 @@ void launch_col_mode(const Params& p, bool causal, hipStream_t s) {
   else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, MODE>), grid, block, 0, s, p);
 }
 
+template <int DT, int KS, int MODE, int NG>
+void launch_col_small_groups(const Params& p, bool causal, hipStream_t s) {
+  const dim3 grid(p.total), block(kThreads);
+  if (causal) hipLaunchKernelGGL((col_small_kernel<DT, KS, true, MODE, NG>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((col_small_kernel<DT, KS, false, MODE, NG>), grid, block, 0, s, p);
+}
+
 template <int DT, int KS, int MODE>
 void launch_col_small_mode(const Params& p, bool causal, hipStream_t s) {
-  const dim3 grid(p.total), block(kThreads);
-  if (causal) hipLaunchKernelGGL((col_small_kernel<DT, KS, true, MODE>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((col_small_kernel<DT, KS, false, MODE>), grid, block, 0, s, p);
+  if (p.M <= 64) launch_col_small_groups<DT, KS, MODE, 4>(p, causal, s);
+  else launch_col_small_groups<DT, KS, MODE, 8>(p, causal, s);
 }
 
 template <int DT, int KS>
@@ -1184,14 +1193,18 @@ int col_reduce_any(const void* q, const void* k, const float* lse, float* out, f
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (M <= kSmallRows && ksteps <= 4) {
     // Few queries: the sweep with all of them resident in every wave and the keys streamed, if the
-    // problem fills the chip that way: about 1024 workgroups, each sweeping at least 16 chunks of keys.
+    // problem fills the chip that way: 512 to 1024 workgroups (at least two per CU), each sweeping at
+    // least 16 chunks of keys, or 8 if that is what it takes.
     const int64_t nchunks = ((int64_t)N + kChunk - 1) / kChunk;
-    int64_t splits = 1024 / p.bh_count;
-    if (splits > nchunks / 16) splits = nchunks / 16;
-    if (splits < 1) splits = 1;
-    const int64_t per = (nchunks + splits - 1) / splits;
-    splits = (nchunks + per - 1) / per;  // no empty ranges
-    if (p.bh_count * splits >= 128 && nchunks >= 16) {
+    int64_t splits = 0;
+    for (int64_t least = 16; least >= 8 && p.bh_count * splits < 512; least /= 2) {  // longer sweeps first
+      splits = 1024 / p.bh_count;
+      if (splits > nchunks / least) splits = nchunks / least;
+      if (splits < 1) splits = 1;
+      const int64_t per = (nchunks + splits - 1) / splits;
+      splits = (nchunks + per - 1) / per;  // no empty ranges
+    }
+    if (p.bh_count * splits >= 512) {
       p.splits = (int)splits;
       p.total = (int)(p.bh_count * splits);
       p.group = head_group(p.bh_count, splits, false);

@@ -220,13 +220,15 @@ def test_at_most_64_queries(m, n, d, causal, dtype):
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("b,h,m,n,d", [
     (4, 16, 64, 4100, 128),    # 64 pairs x 4 key ranges
-    (1, 130, 33, 1030, 64),    # one range per pair, a ragged last chunk, padded query groups
-    (2, 40, 1, 2048, 16),      # a single query
-    (3, 50, 64, 1100, 72),     # D not a multiple of 32
+    (2, 130, 33, 1030, 64),    # one range per pair, a ragged last chunk, padded query groups
+    (4, 40, 1, 2048, 16),      # a single query
+    (6, 50, 64, 1100, 72),     # D not a multiple of 32
     (1, 8, 17, 40000, 32),     # many ranges per pair
+    (4, 16, 128, 4100, 128),   # eight resident query groups
+    (4, 70, 97, 1030, 48),     # eight groups, the last two partly / wholly padding
 ])
 def test_few_queries_with_streamed_keys(b, h, m, n, d, causal, dtype):
-    """At most 64 queries, D <= 128 and enough (b,h) pairs x keys to fill the chip: the column
+    """At most 128 queries, D <= 128 and enough (b,h) pairs x keys to fill the chip: the column
     sweep with the queries resident in every wave and the keys streamed in ranges; sum, mean, max and
     the fused sum+max form.  With the mask the diagonal is the last M keys."""
     q, k = _inputs.randn_pair(b, h, m, n, d, seed=b * h + m + n, dtype=dtype)
