@@ -53,11 +53,19 @@ inline int64_t rows_swept(int M, int nb) {
   const int waves = rem ? (rem + 31) / 32 : 0;   // blocks of the last tile that hold queries
   return (int64_t)(M / trows) * trows + (waves < kWaves ? waves : kWaves) * 32 * nb;
 }
-inline int row_blocks_per_wave(int ksteps, int M) {
+// One block also wins when two would give between one and two workgroups per CU (with fewer than
+// one the keys of a tile are split over workgroups instead, see row_splits; that case does not depend
+// on `causal`, so the size of the lse buffer does not either).  With the mask exactly two per CU is
+// still too coarse: the chip then waits for the workgroup with the longest sweep.
+inline int row_blocks_per_wave(int ksteps, int M, int64_t bh, bool causal) {
   if (ksteps > 4) return 1;
-  return rows_swept(M, 1) * (100 + 3 * ksteps) < rows_swept(M, 2) * 100 ? 1 : 2;
+  if (rows_swept(M, 1) * (100 + 3 * ksteps) < rows_swept(M, 2) * 100) return 1;
+  const int64_t wgs2 = bh * ((M + kWaves * 64 - 1) / (kWaves * 64));
+  return (wgs2 >= 256 && wgs2 < 512 + (causal ? 1 : 0)) ? 1 : 2;
 }
-inline int row_tile_rows(int ksteps, int M) { return kWaves * 32 * row_blocks_per_wave(ksteps, M); }
+inline int row_tile_rows(int ksteps, int M, int64_t bh, bool causal) {
+  return kWaves * 32 * row_blocks_per_wave(ksteps, M, bh, causal);
+}
 constexpr int kMaxKSteps = 8;                 // D <= 256
 constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row sub-steps)
 constexpr float kNegInf = -__builtin_inff();
@@ -599,11 +607,19 @@ struct LsePair {
 __host__ __device__ constexpr int col_blocks_per_wave(int ksteps, int mode) {
   return mode == kModeBoth ? 1 : blocks_per_wave(ksteps);
 }
+// Blocks per wave the host asks for: with the mask, between one and two workgroups per CU of 256 keys
+// are too coarse (the chip waits for the longest sweep), so those launches use 128-key tiles.
+inline int col_tile_blocks(int ksteps, int mode, int N, int64_t bh, bool causal) {
+  const int nb = col_blocks_per_wave(ksteps, mode);
+  if (nb == 1 || !causal) return nb;
+  const int64_t wgs2 = bh * ((N + kWaves * 64 - 1) / (kWaves * 64));
+  return (wgs2 >= 256 && wgs2 <= 512) ? 1 : 2;
+}
 
-template <int DT, int KS, bool CAUSAL, int MODE>
+template <int DT, int KS, bool CAUSAL, int MODE, int NB>
 __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p) {
   using St = Stager<KS>;
-  constexpr int NB = col_blocks_per_wave(KS, MODE), NG = 2 * NB;
+  constexpr int NG = 2 * NB;
   constexpr int kTileRows = kWaves * 32 * NB;
   constexpr int kStage = St::kBytes + kChunk * 4;     // rows + their lse
   constexpr int kRed = kWaves * NG * 4 * 64 * 4;      // end-of-sweep transpose buffer
@@ -1008,14 +1024,15 @@ int head_group(int64_t bh, int64_t per_bh, bool causal) {
 }
 
 int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H, int M, int N, int D,
-                const int64_t qs[4], const int64_t ks[4], float scale, bool by_keys, int col_mode = kModeSum) {
+                const int64_t qs[4], const int64_t ks[4], float scale, bool by_keys, bool causal,
+                int col_mode = kModeSum) {
   if (!q || !k || !qs || !ks) return fail(FCR_E_NULL, "null pointer argument");
   if (dtype != FCR_DTYPE_F16 && dtype != FCR_DTYPE_BF16) return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16 or FCR_DTYPE_BF16");
   if (B < 1 || H < 1 || M < 1 || N < 1) return fail(FCR_E_SHAPE, "B, H, M, N must be >= 1");
   if (D < 8 || D > 32 * kMaxKSteps || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 256]");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
-  const int trows = by_keys ? kWaves * 32 * col_blocks_per_wave((D + 31) / 32, col_mode) : row_tile_rows((D + 31) / 32, M);
+  const int trows = by_keys ? kWaves * 32 * col_tile_blocks((D + 31) / 32, col_mode, N, bh, causal) : row_tile_rows((D + 31) / 32, M, bh, causal);
   const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
   if (bh * tiles > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
   if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
@@ -1047,7 +1064,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
 // workgroup per CU; otherwise the keys of a tile are split so that about two per CU run, each
 // keeping at least four 64-key chunks.
 int row_splits(int B, int H, int M, int N, int D) {
-  const int trows = row_tile_rows((D + 31) / 32, M);
+  const int trows = row_tile_rows((D + 31) / 32, M, (int64_t)B * H, false);  // same with the mask when wgs < 256
   const int64_t wgs = (int64_t)B * H * ((M + trows - 1) / trows);
   const int64_t chunks = (N + kChunk - 1) / kChunk;
   if (wgs >= 256 || chunks < 16) return 1;
@@ -1074,7 +1091,7 @@ void launch_lse_blocks(const Params& p, bool causal, hipStream_t s) {
 template <int DT, int KS>
 void launch_lse(const Params& p, bool causal, hipStream_t s) {
   if constexpr (KS <= 4) {
-    if (row_blocks_per_wave(KS, p.M) == 2) return launch_lse_blocks<DT, KS, 2, false>(p, causal, s);
+    if (row_blocks_per_wave(KS, p.M, p.bh_count, causal) == 2) return launch_lse_blocks<DT, KS, 2, false>(p, causal, s);
   }
   // one row tile per (b,h) and at least 1 GiB of keys: stream them past the caches
   const int64_t key_bytes = (int64_t)p.bh_count * p.N * p.dgran * 16;
@@ -1085,8 +1102,16 @@ void launch_lse(const Params& p, bool causal, hipStream_t s) {
 template <int DT, int KS, int MODE>
 void launch_col_mode(const Params& p, bool causal, hipStream_t s) {
   const dim3 grid(p.total), block(kThreads);
-  if (causal) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, MODE>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, MODE>), grid, block, 0, s, p);
+  constexpr int NB = col_blocks_per_wave(KS, MODE);
+  if constexpr (NB == 2) {
+    // the finer tiles only exist with the mask (see col_tile_blocks)
+    if (causal && col_tile_blocks(KS, MODE, p.N, p.bh_count, true) == 1) {
+      hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, MODE, 1>), grid, block, 0, s, p);
+      return;
+    }
+  }
+  if (causal) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, MODE, NB>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, MODE, NB>), grid, block, 0, s, p);
 }
 
 template <int DT, int KS, int MODE, int NG>
@@ -1156,7 +1181,7 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
                 void* stream) {
   Params p;
   if (!lse) return fail(FCR_E_NULL, "null pointer argument");
-  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, false);
+  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, false, causal != 0);
   if (rc) return rc;
   p.lse = lse;
   p.splits = row_splits(B, H, M, N, D);
@@ -1183,7 +1208,7 @@ int col_reduce_any(const void* q, const void* k, const float* lse, float* out, f
                    float scale, int causal, void* stream) {
   Params p;
   if (!lse || !out || (mode == kModeBoth && !out2)) return fail(FCR_E_NULL, "null pointer argument");
-  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true, mode);
+  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true, causal != 0, mode);
   if (rc) return rc;
   p.group = head_group(p.bh_count, p.tiles, causal != 0);
   p.lse = const_cast<float*>(lse);

@@ -238,6 +238,20 @@ def test_few_queries_with_streamed_keys(b, h, m, n, d, causal, dtype):
     check(got[1], colreduce_ref(q, k, "max", causal), "max", "streamed keys fused")
 
 
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("b,h,m,n,d", [
+    (1, 32, 2048, 2048, 128),   # 256 workgroups of 256 rows either way: both sweeps take 128-row tiles
+    (4, 16, 300, 1100, 64),     # only the column sweep is in that range
+    (2, 8, 8192, 520, 32),      # only the row sweep is; M > N
+    (1, 16, 8192, 8192, 16),    # exactly two per CU: finer tiles with the mask only
+])
+def test_between_one_and_two_workgroups_per_cu(b, h, m, n, d, causal):
+    """Launches that would put between one and two 256-row workgroups on a CU use 128-row tiles (the
+    column sweep only with the mask)."""
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=m + n + d)
+    run_all(q, k, causal, what=f"finer tiles b{b} h{h} m{m} n{n} d{d}", reductions=("sum", "max"))
+
+
 @pytest.mark.parametrize("m", [100, 128, 300, 384, 600])
 def test_row_sweep_block_choice(m):
     """Query counts for which the row sweep keeps one 32-row block per wave (M <= 128 and ragged M
