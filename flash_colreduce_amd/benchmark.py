@@ -1,6 +1,6 @@
 """Latency / peak-memory sweep over the reference's 20 benchmark shapes.
 
-    python -m flash_colreduce_amd.benchmark [--budget SECONDS] [--no-naive] [--out FILE]
+    python -m flash_colreduce_amd.benchmark [--budget SECONDS] [--no-naive] [--rows 0,13] [--out FILE]
 
 Same shapes and method as the reference's harness (benchmarks/run.py:11-92): fp16, H = 32, D = 128,
 reduction = "sum"; per implementation one call, a 10-call calibration, then `iters` warm-up calls and
@@ -55,7 +55,7 @@ def measure_memory(fn) -> float:
     return torch.cuda.max_memory_allocated() / 2**20
 
 
-def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout):
+def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None):
     name = torch.cuda.get_device_name(0)
     print(f"Benchmark results on {name} (fp16, reduction=sum)", file=out)
     head = (f"{'configuration':<48} {'flash ms':>10} {'naive ms':>10} {'speedup':>8} {'flash MB':>10} "
@@ -64,7 +64,9 @@ def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout):
     print("-" * len(head), file=out)
     rows = []
     with torch.inference_mode():
-        for cfg in CONFIGS:
+        for index, cfg in enumerate(CONFIGS):
+            if only is not None and index not in only:
+                continue
             b, h, m, n, d, causal = (cfg[k] for k in ("b", "h", "m", "n", "d", "is_causal"))
             g = torch.Generator(device="cuda").manual_seed(0)
             q = torch.randn(b, h, m, d, device="cuda", dtype=torch.float16, generator=g)
@@ -94,16 +96,18 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--budget", type=float, default=2.0, help="seconds of timed calls per implementation")
     ap.add_argument("--no-naive", action="store_true", help="skip the materialising implementation")
+    ap.add_argument("--rows", default=None, help="comma separated indices (0..19) of the shapes to run; default all")
     ap.add_argument("--out", default=None, help="also write the table to this file")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("benchmark needs a GPU")
+    only = None if args.rows is None else {int(r) for r in args.rows.split(",")}
     if args.out:
         with open(args.out, "w") as f:
-            run(args.budget, not args.no_naive, out=f)
+            run(args.budget, not args.no_naive, out=f, only=only)
         print(open(args.out).read())
     else:
-        run(args.budget, not args.no_naive)
+        run(args.budget, not args.no_naive, only=only)
 
 
 if __name__ == "__main__":
