@@ -607,13 +607,15 @@ struct LsePair {
 __host__ __device__ constexpr int col_blocks_per_wave(int ksteps, int mode) {
   return mode == kModeBoth ? 1 : blocks_per_wave(ksteps);
 }
-// Blocks per wave the host asks for: with the mask, between one and two workgroups per CU of 256 keys
-// are too coarse (the chip waits for the longest sweep), so those launches use 128-key tiles.
+// Blocks per wave the host asks for.  Strictly between one and two workgroups of 256 keys per CU
+// leave CUs unevenly loaded, and with the mask one or two per CU are too coarse as well (the chip
+// waits for the longest sweep): those launches use 128-key tiles.
 inline int col_tile_blocks(int ksteps, int mode, int N, int64_t bh, bool causal) {
   const int nb = col_blocks_per_wave(ksteps, mode);
-  if (nb == 1 || !causal) return nb;
+  if (nb == 1) return nb;
   const int64_t wgs2 = bh * ((N + kWaves * 64 - 1) / (kWaves * 64));
-  return (wgs2 >= 256 && wgs2 <= 512) ? 1 : 2;
+  if (causal) return (wgs2 >= 256 && wgs2 <= 512) ? 1 : 2;
+  return (wgs2 > 256 && wgs2 < 512) ? 1 : 2;
 }
 
 template <int DT, int KS, bool CAUSAL, int MODE, int NB>
@@ -1104,9 +1106,9 @@ void launch_col_mode(const Params& p, bool causal, hipStream_t s) {
   const dim3 grid(p.total), block(kThreads);
   constexpr int NB = col_blocks_per_wave(KS, MODE);
   if constexpr (NB == 2) {
-    // the finer tiles only exist with the mask (see col_tile_blocks)
-    if (causal && col_tile_blocks(KS, MODE, p.N, p.bh_count, true) == 1) {
-      hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, MODE, 1>), grid, block, 0, s, p);
+    if (col_tile_blocks(KS, MODE, p.N, p.bh_count, causal) == 1) {
+      if (causal) hipLaunchKernelGGL((col_reduce_kernel<DT, KS, true, MODE, 1>), grid, block, 0, s, p);
+      else hipLaunchKernelGGL((col_reduce_kernel<DT, KS, false, MODE, 1>), grid, block, 0, s, p);
       return;
     }
   }

@@ -244,10 +244,11 @@ def test_few_queries_with_streamed_keys(b, h, m, n, d, causal, dtype):
     (4, 16, 300, 1100, 64),     # only the column sweep is in that range
     (2, 8, 8192, 520, 32),      # only the row sweep is; M > N
     (1, 16, 8192, 8192, 16),    # exactly two per CU: finer tiles with the mask only
+    (1, 32, 512, 2880, 128),    # 384 column workgroups of 256 keys: finer tiles without the mask too
 ])
 def test_between_one_and_two_workgroups_per_cu(b, h, m, n, d, causal):
-    """Launches that would put between one and two 256-row workgroups on a CU use 128-row tiles (the
-    column sweep only with the mask)."""
+    """Launches that would put between one and two 256-row workgroups on a CU use 128-row tiles (at
+    exactly one or two per CU depending on the sweep and the mask)."""
     q, k = _inputs.randn_pair(b, h, m, n, d, seed=m + n + d)
     run_all(q, k, causal, what=f"finer tiles b{b} h{h} m{m} n{n} d{d}", reductions=("sum", "max"))
 
