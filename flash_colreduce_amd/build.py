@@ -36,10 +36,6 @@ def hipcc_path() -> str:
     return exe
 
 
-TOOL_SRC = os.path.join(HERE, "csrc", "tools", "mfma_rate.hip")
-TOOL = os.path.join(HERE, "mfma_rate")
-
-
 def build(verbose: bool = True, extra_flags=()) -> str:
     cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, SRC, "-o", LIB]
     if verbose:
@@ -48,19 +44,5 @@ def build(verbose: bool = True, extra_flags=()) -> str:
     return LIB
 
 
-def build_tools(verbose: bool = True) -> str:
-    """Diagnostics that are not part of the library (MFMA rate under random operands)."""
-    cmd = [hipcc_path(), "-O3", "--offload-arch=gfx950", "-Xclang", "-target-feature", "-Xclang",
-           "-packed-fp32-ops", TOOL_SRC, "-o", TOOL]
-    if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
-    return TOOL
-
-
 if __name__ == "__main__":
-    args = sys.argv[1:]
-    if "--tools" in args:
-        args.remove("--tools")
-        build_tools()
-    build(extra_flags=args)
+    build(extra_flags=sys.argv[1:])

@@ -42,6 +42,26 @@ constexpr int kThreads = kWaves * 64;
 // two 32-row blocks (four groups) while their fragments fit the register file next to the
 // accumulators (D <= 128: 4 k-steps), one block for larger D.  A workgroup keeps 4 * 32 * blocks rows.
 __host__ __device__ constexpr int blocks_per_wave(int ksteps) { return ksteps <= 4 ? 2 : 1; }
+// Compute units of the current device, asked once per device.  The tile, split and group choices below
+// are stated in workgroups per CU (these kernels run two per CU).  256, an MI355X in its default
+// partition mode, when no device can be asked (argument checks on a host without a GPU).
+inline int chip_cus() {
+  static int cached[64] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return 256;
+  }
+  int n = __atomic_load_n(&cached[dev], __ATOMIC_RELAXED);
+  if (n == 0) {
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n < 1) {
+      (void)hipGetLastError();
+      n = 256;
+    }
+    __atomic_store_n(&cached[dev], n, __ATOMIC_RELAXED);
+  }
+  return n;
+}
 // The row kernel has both forms for D <= 128 and the host picks per problem.  Waves whose rows are all
 // padding do no arithmetic, so a launch costs (rows in waves with at least one query) x (cost per
 // row); one block per wave costs about 3 % per k-step more per row (every streamed fragment feeds
@@ -61,7 +81,8 @@ inline int row_blocks_per_wave(int ksteps, int M, int64_t bh, bool causal) {
   if (ksteps > 4) return 1;
   if (rows_swept(M, 1) * (100 + 3 * ksteps) < rows_swept(M, 2) * 100) return 1;
   const int64_t wgs2 = bh * ((M + kWaves * 64 - 1) / (kWaves * 64));
-  return (wgs2 >= 256 && wgs2 < 512 + (causal ? 1 : 0)) ? 1 : 2;
+  const int cus = chip_cus();
+  return (wgs2 >= cus && wgs2 < 2 * cus + (causal ? 1 : 0)) ? 1 : 2;
 }
 inline int row_tile_rows(int ksteps, int M, int64_t bh, bool causal) {
   return kWaves * 32 * row_blocks_per_wave(ksteps, M, bh, causal);
@@ -614,8 +635,9 @@ inline int col_tile_blocks(int ksteps, int mode, int N, int64_t bh, bool causal)
   const int nb = col_blocks_per_wave(ksteps, mode);
   if (nb == 1) return nb;
   const int64_t wgs2 = bh * ((N + kWaves * 64 - 1) / (kWaves * 64));
-  if (causal) return (wgs2 >= 256 && wgs2 <= 512) ? 1 : 2;
-  return (wgs2 > 256 && wgs2 < 512) ? 1 : 2;
+  const int cus = chip_cus();
+  if (causal) return (wgs2 >= cus && wgs2 <= 2 * cus) ? 1 : 2;
+  return (wgs2 > cus && wgs2 < 2 * cus) ? 1 : 2;
 }
 
 template <int DT, int KS, bool CAUSAL, int MODE, int NB>
@@ -998,7 +1020,7 @@ int fail(int code, const char* what) {
   return code;
 }
 
-int check_strides(const void* ptr, const int64_t s[4], const char* name) {
+int check_strides(const void* ptr, const int64_t s[4], const char* name, int rows, int D) {
   if (s[3] != 1) {
     snprintf(g_err, sizeof(g_err), "%s: stride of the last dimension must be 1 (got %lld)", name, (long long)s[3]);
     return FCR_E_STRIDE;
@@ -1010,6 +1032,13 @@ int check_strides(const void* ptr, const int64_t s[4], const char* name) {
              name);
     return FCR_E_STRIDE;
   }
+  // Rows that overlap (an expanded operand has row stride 0) cannot be described by the buffer views
+  // the kernels read through: the view of the rows from r on is (rows - r) * stride bytes long.
+  if (rows > 1 && s[2] < D) {
+    snprintf(g_err, sizeof(g_err), "%s: row stride (%lld) must be at least D (%d) when there is more than one row",
+             name, (long long)s[2], D);
+    return FCR_E_STRIDE;
+  }
   return 0;
 }
 
@@ -1019,7 +1048,8 @@ int check_strides(const void* ptr, const int64_t s[4], const char* name) {
 // never fewer than 32 pairs (measured: smaller groups lose up to 8 % on 32 heads of 8192 rows,
 // larger ones up to 11 % on 1024 heads of 2048 rows, whose operands then come from HBM per tile).
 int head_group(int64_t bh, int64_t per_bh, bool causal) {
-  int64_t g = ((causal ? 1024 : 256) / per_bh) & ~7ll;
+  const int cus = chip_cus();
+  int64_t g = ((causal ? 4 * cus : cus) / per_bh) & ~7ll;
   const int64_t least = causal ? 32 : 8;
   if (g < least) g = least;
   return (int)(g < bh ? g : bh);
@@ -1034,14 +1064,15 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   if (D < 8 || D > 32 * kMaxKSteps || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 256]");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
+  if (bh * (((int64_t)(by_keys ? N : M) + 127) / 128) > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
+  if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
+  int rc = check_strides(q, qs, "q", M, D);
+  if (rc) return rc;
+  rc = check_strides(k, ks, "k", N, D);
+  if (rc) return rc;
+  // the device is first asked (for its CU count) here, after every argument check
   const int trows = by_keys ? kWaves * 32 * col_tile_blocks((D + 31) / 32, col_mode, N, bh, causal) : row_tile_rows((D + 31) / 32, M, bh, causal);
   const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
-  if (bh * tiles > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
-  if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
-  int rc = check_strides(q, qs, "q");
-  if (rc) return rc;
-  rc = check_strides(k, ks, "k");
-  if (rc) return rc;
   p.q = static_cast<const char*>(q);
   p.k = static_cast<const char*>(k);
   p.q_sb = qs[0] * 2; p.q_sh = qs[1] * 2; p.q_sr = qs[2] * 2;
@@ -1069,8 +1100,9 @@ int row_splits(int B, int H, int M, int N, int D) {
   const int trows = row_tile_rows((D + 31) / 32, M, (int64_t)B * H, false);  // same with the mask when wgs < 256
   const int64_t wgs = (int64_t)B * H * ((M + trows - 1) / trows);
   const int64_t chunks = (N + kChunk - 1) / kChunk;
-  if (wgs >= 256 || chunks < 16) return 1;
-  int64_t s = 512 / wgs;
+  const int cus = chip_cus();
+  if (wgs >= cus || chunks < 16) return 1;
+  int64_t s = 2 * cus / wgs;
   if (s > chunks / 4) s = chunks / 4;
   if (s > 64) s = 64;
   return s < 1 ? 1 : (int)s;
@@ -1224,14 +1256,15 @@ int col_reduce_any(const void* q, const void* k, const float* lse, float* out, f
     // least 16 chunks of keys, or 8 if that is what it takes.
     const int64_t nchunks = ((int64_t)N + kChunk - 1) / kChunk;
     int64_t splits = 0;
-    for (int64_t least = 16; least >= 8 && p.bh_count * splits < 512; least /= 2) {  // longer sweeps first
-      splits = 1024 / p.bh_count;
+    const int cus = chip_cus();
+    for (int64_t least = 16; least >= 8 && p.bh_count * splits < 2 * cus; least /= 2) {  // longer sweeps first
+      splits = 4 * cus / p.bh_count;
       if (splits > nchunks / least) splits = nchunks / least;
       if (splits < 1) splits = 1;
       const int64_t per = (nchunks + splits - 1) / splits;
       splits = (nchunks + per - 1) / per;  // no empty ranges
     }
-    if (p.bh_count * splits >= 512) {
+    if (p.bh_count * splits >= 2 * cus) {
       p.splits = (int)splits;
       p.total = (int)(p.bh_count * splits);
       p.group = head_group(p.bh_count, splits, false);

@@ -6,7 +6,6 @@ a C ABI (include/fcr.h); torch is used for device memory and the current stream 
 """
 from __future__ import annotations
 
-import functools
 import math
 from typing import Optional
 
@@ -52,7 +51,8 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
         return torch.nn.functional.pad(x, (0, 8 - d % 8))  # new contiguous tensor
     ok = (x.stride(3) == 1 and x.data_ptr() % 16 == 0 and
           all(x.stride(i) % 8 == 0 and x.stride(i) >= 0 for i in (0, 1, 2)) and
-          x.stride(2) < (1 << 24))
+          x.stride(2) < (1 << 24) and
+          (x.shape[2] <= 1 or x.stride(2) >= d))  # rows must not overlap (expand() gives stride 0)
     if ok:
         return x
     # a contiguous tensor can still start at a misaligned address: contiguous() would hand it back
@@ -128,10 +128,12 @@ def _launch(query, key, kinds, is_causal, scale):
     return outs, lse[: b * h * m]
 
 
-@functools.lru_cache(maxsize=8)
 def _countdown(count: int, device: torch.device) -> torch.Tensor:
-    """count, count-1, .., 1: the causal mean divisor from the offset on (flash.py:381-382), kept
-    between calls because building it costs more host time than a small problem's kernels."""
+    """count, count-1, .., 1: the causal mean divisor from the offset on (flash.py:381-382).
+
+    Built on the device by every call, on the caller's stream.  A tensor kept between calls would be
+    wrong under HIP graph capture (its fill would only be recorded, and its memory would belong to the
+    graph's pool) and would be shared between streams without an event."""
     return torch.arange(count, 0, -1, device=device)
 
 

@@ -26,7 +26,8 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_lib.LIB_PATH)
     names = _declared_symbols()
     assert {"fcr_version", "fcr_last_error", "fcr_lse_bytes", "fcr_row_lse", "fcr_col_reduce",
-            "fcr_col_reduce_sum_max", "fcr_pack_f32", "fcr_colreduce"} <= set(names)
+            "fcr_col_reduce_sum_max", "fcr_pack_f32", "fcr_colreduce",
+            "fcr_topk_mask"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
 
@@ -65,6 +66,7 @@ def test_c_abi_rejects_bad_arguments_without_a_device(fn):
         (dict(D=264), -3), (dict(M=(1 << 30) + 1), -3),
         (dict(qs=(512, 512, 64, 2)), -4), (dict(ks=(512, 512, 60, 1)), -4), (dict(q=18), -4),
         (dict(ks=(512, -512, 64, 1)), -4),
+        (dict(qs=(512, 512, 0, 1)), -4), (dict(ks=(512, 512, 32, 1)), -4),   # overlapping rows
         (dict(scale=float("inf")), -6), (dict(scale=float("nan")), -6),
     ]
     if fn != "row_lse":

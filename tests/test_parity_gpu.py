@@ -311,6 +311,39 @@ def test_strided_inputs(causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+def test_expanded_operands(causal):
+    """Operands whose rows overlap in memory (expand() gives a row stride of 0): the library's buffer
+    views cannot describe them, so the host copies; one query repeated M times, one key repeated N
+    times, and a batch/head broadcast (stride 0 on those dimensions is addressed directly)."""
+    b, h, m, n, d = 2, 3, 70, 200, 64
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=61)
+    qd, kd = q.cuda(), k.cuda()
+
+    def run(qx, kx, what):  # expanded on the device: a host-to-device copy would make them dense
+        assert qx.is_cuda and kx.is_cuda
+        for red in REDUCTIONS:
+            got = fca.flash_colreduce(qx, kx, red, is_causal=causal, out_dtype=torch.float32)
+            check(got, colreduce_ref(qx.cpu(), kx.cpu(), red, causal), red, what)
+
+    q1 = qd[:, :, :1].expand(b, h, m, d)
+    assert q1.stride(2) == 0
+    run(q1, kd, "expanded query rows")
+    k1 = kd[:, :, 3:4].expand(b, h, n, d)
+    run(qd, k1, "expanded key rows")
+    kb = kd[:1, :1].expand(b, h, n, d)
+    assert kb.stride(0) == 0 and kb.stride(1) == 0
+    run(qd, kb, "key broadcast over batch and heads")
+    # through the C ABI the overlapping rows are rejected, not misread
+    from flash_colreduce_amd import _lib
+    lib = _lib.load()
+    out = torch.empty(b * h, n, device="cuda")
+    lse = torch.empty(lib.fcr_lse_bytes(b, h, m, n, d) // 4, device="cuda")
+    rc = lib.fcr_colreduce(q1.data_ptr(), kd.data_ptr(), out.data_ptr(), lse.data_ptr(), _lib.DTYPE_F16, b, h, m, n, d,
+                           _lib.strides4(q1.stride()), _lib.strides4(kd.stride()), 0.125, 0, int(causal), None)
+    assert rc == -4 and b"row stride" in lib.fcr_last_error()
+
+
+@pytest.mark.parametrize("causal", [False, True])
 def test_score_jumps_renormalise(causal):
     """Scores that jump by far more than 64 binades in the middle of the sweep, and rows whose
     scores are all hugely negative: exercises the renormalisation of the running row sum."""
@@ -497,6 +530,38 @@ def test_hip_graph_capture_and_replay():
         torch.cuda.synchronize()
         assert torch.equal(got[0], es) and torch.equal(got[1], em) and torch.equal(got[2], e1), seed
         check(got[0], colreduce_ref(q1, k1, "sum", True), "sum", f"graph replay seed {seed}")
+
+
+def test_graph_capture_of_a_causal_mean_never_seen_before():
+    """The causal mean divisor is built on the device by every call.  Capture a causal mean whose
+    divisor length was never used in this process, call eagerly BEFORE the first replay, then capture a
+    second graph with the same length and replay only that one: each result must be the oracle's."""
+    b, h, m, n, d = 1, 3, 211, 347, 32      # divisor length 211, used by no other test
+    qc, kc = _inputs.randn_pair(b, h, m, n, d, seed=91)
+    q, k = qc.cuda(), kc.cuda()
+    want = colreduce_ref(qc, kc, "mean", True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):  # warm up the kernels, but not the mean epilogue
+        fca.flash_colreduce(q, k, "sum", True, out_dtype=torch.float32)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g1 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g1):
+        out1 = fca.flash_colreduce(q, k, "mean", True, out_dtype=torch.float32)
+    eager = fca.flash_colreduce(q, k, "mean", True, out_dtype=torch.float32)   # before any replay
+    torch.cuda.synchronize()
+    check(eager, want, "mean", "eager call between capture and first replay")
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2):
+        out2 = fca.flash_colreduce(q, k, "mean", True, out_dtype=torch.float32)
+    g2.replay()                                                                  # g1 never replayed so far
+    torch.cuda.synchronize()
+    check(out2, want, "mean", "second graph replayed alone")
+    assert torch.equal(out2, eager)
+    g1.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(out1, eager)
 
 
 def test_launcher_stub_of_the_integration_notes():
