@@ -53,6 +53,9 @@ def _declare(lib):
     lib.fcr_colreduce.restype = c.c_int
     lib.fcr_colreduce.argtypes = ([c.c_void_p, c.c_void_p, c.c_void_p, c.c_void_p] + common +
                                   [c.c_int, c.c_int, c.c_void_p])
+    lib.fcr_colreduce_static.restype = c.c_int
+    lib.fcr_colreduce_static.argtypes = ([c.c_void_p, c.c_void_p, c.c_void_p] + common +
+                                         [c.c_int, c.c_int, c.c_void_p])
     return lib
 
 

@@ -1334,4 +1334,59 @@ int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int d
                         causal, stream);
 }
 
+// Scratch of fcr_colreduce_static: the row statistics and, for few query rows against many keys, the
+// partial results of the split row sweep.  One copy per GPU, held until the process ends.  Host code
+// must not pass the array's name to a kernel (it is a host-side stand-in there): the device address is
+// asked once per device and kept.
+static __device__ __align__(256) unsigned char scratch[FCR_STATIC_SCRATCH_BYTES];
+
+namespace {
+int static_scratch(float** ptr) {
+  static void* ptrs[64] = {};
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) {
+    snprintf(g_err, sizeof(g_err), "hipGetDevice failed: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  if (dev < 0 || dev >= 64) return fail(FCR_E_SHAPE, "device ordinal must be below 64");
+  void* p = __atomic_load_n(&ptrs[dev], __ATOMIC_ACQUIRE);
+  if (!p) {
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));  // this device's copy of the array
+    if (e != hipSuccess || !p) {
+      snprintf(g_err, sizeof(g_err), "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+      return e != hipSuccess ? (int)e : (int)hipErrorInvalidSymbol;
+    }
+    __atomic_store_n(&ptrs[dev], p, __ATOMIC_RELEASE);
+  }
+  *ptr = static_cast<float*>(p);
+  return 0;
+}
+}  // namespace
+
+int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, int B, int H, int M, int N, int D,
+                         const int64_t q_strides[4], const int64_t k_strides[4], float scale, int reduction,
+                         int causal, void* stream) {
+  if (!out) return fail(FCR_E_NULL, "null pointer argument");
+  if (reduction != FCR_REDUCE_SUM && reduction != FCR_REDUCE_MAX)
+    return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM or FCR_REDUCE_MAX");
+  // every argument check of the two kernels, before the device is asked for anything
+  Params p;
+  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, false, causal != 0);
+  if (rc) return rc;
+  const size_t need = fcr_lse_bytes(B, H, M, N, D);
+  if (need > (size_t)FCR_STATIC_SCRATCH_BYTES) {
+    snprintf(g_err, sizeof(g_err),
+             "fcr_colreduce_static: this problem needs %zu bytes of scratch, the built-in buffer has %zu; "
+             "use fcr_colreduce with a caller-provided buffer",
+             need, (size_t)FCR_STATIC_SCRATCH_BYTES);
+    return FCR_E_SCRATCH;
+  }
+  float* ws = nullptr;
+  rc = static_scratch(&ws);
+  if (rc) return rc;
+  // Both kernels write every value of the buffer they later read, so nothing has to be cleared.
+  return fcr_colreduce(q, k, out, ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, reduction, causal, stream);
+}
+
 }  // extern "C"

@@ -56,6 +56,10 @@ extern "C" {
 #define FCR_E_STRIDE -4    /* d stride != 1 or a stride / base pointer breaks 16-byte alignment */
 #define FCR_E_REDUCTION -5 /* reduction is not FCR_REDUCE_* */
 #define FCR_E_SCALE -6     /* scale is not finite */
+#define FCR_E_SCRATCH -7   /* fcr_colreduce_static: the problem needs more than FCR_STATIC_SCRATCH_BYTES */
+
+/* size of the built-in scratch buffer of fcr_colreduce_static, per GPU */
+#define FCR_STATIC_SCRATCH_BYTES (16u << 20)
 
 /* Library version (FCR_VERSION it was built from). */
 int fcr_version(void);
@@ -127,6 +131,23 @@ int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, in
 int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H,
                   int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
                   float scale, int reduction, int causal, void* stream);
+
+/*
+ * fcr_colreduce without the lse_ws argument, for callers that cannot allocate device memory (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference, whose launcher allocates with torch on every call (flash.py:286).  The row statistics and
+ * the split row sweep's partial results live in a buffer of FCR_STATIC_SCRATCH_BYTES that is part of
+ * the library's device image: every GPU the library runs on holds one until the process ends.  The call
+ * allocates and frees nothing.  Problems with fcr_lse_bytes(B,H,M,N,D) > FCR_STATIC_SCRATCH_BYTES are
+ * rejected with FCR_E_SCRATCH (16 MiB covers B*H*M <= 4 Mi rows when the keys are not split, e.g.
+ * 32 heads of 131072 queries).  All calls on one GPU share the buffer: calls that overlap in time on one
+ * GPU (different streams or threads) race; calls on one stream are ordered and safe.  The first call on
+ * a device asks the runtime for the buffer's address and should be made outside graph capture.
+ * Results are bitwise those of fcr_colreduce.
+ */
+int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, int B, int H, int M, int N,
+                         int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
+                         int reduction, int causal, void* stream);
 
 #ifdef __cplusplus
 }
