@@ -174,13 +174,13 @@ __device__ __forceinline__ void map_block_split(const Params& p, bool longest_is
 // of four.
 template <int NB>
 __device__ __forceinline__ void wave_groups(int tile, int wave, int (&rows)[2 * NB]) {
-  const int b0 = tile * (kWaves * 32 * NB) + 32 * wave;
-  rows[0] = b0;
-  rows[1] = b0 + 16;
-  if (NB == 2) {
-    const int b1 = tile * (kWaves * 32 * NB) + 32 * (7 - wave);
-    rows[2 * NB - 2] = b1;
-    rows[2 * NB - 1] = b1 + 16;
+  const int t0 = tile * (kWaves * 32 * NB);
+#pragma unroll
+  for (int i = 0; i < NB; ++i) {
+    // blocks w, 7-w (, 8+w, 15-w): even positions count up, odd ones count down inside a run of eight
+    const int blk = (NB == 1) ? wave : 8 * (i / 2) + ((i & 1) ? 7 - wave : wave);
+    rows[2 * i] = t0 + 32 * blk;
+    rows[2 * i + 1] = t0 + 32 * blk + 16;
   }
 }
 
@@ -190,7 +190,7 @@ __device__ __forceinline__ void wave_groups(int tile, int wave, int (&rows)[2 * 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t rows_view(const char* base, int64_t row_bytes, int row0,
                                                             int nrows) {
   int64_t bytes = (int64_t)(nrows - row0) * row_bytes;
-  bytes = bytes < 0 ? 0 : (bytes > 0xffffffffll ? 0xffffffffll : bytes);
+  bytes = bytes < 0 ? 0 : (bytes > 0xfffffff0ll ? 0xfffffff0ll : bytes);
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<char*>(base) + (int64_t)row0 * row_bytes, 0,
                                            (int)(uint32_t)bytes, 0x00020000);
 }
@@ -222,60 +222,90 @@ __device__ __forceinline__ void load_resident(u32x4 (&f)[NG][KS], const char* ba
   }
 }
 
-// Global -> registers -> LDS staging of kChunk rows of the streamed operand.
-// LDS rows are padded by 32 bytes: a 16-byte fragment read is served in passes of lanes {0-7, 16-23},
-// {8-15, 24-31}, .. (eight consecutive rows at two neighbouring 16-byte columns), and with a pitch of
-// 8 banks modulo 64 these fall into distinct banks (SQ_LDS_BANK_CONFLICT = 0; with 16 bytes of padding
-// every read took two passes).  A thread moves the same granules (row r, 16-byte column cg) of
-// every chunk, so its source offset inside a chunk and its LDS offset are computed once.
-// Granule columns at or past D/8 (the zero padding up to the MFMA k-step) are never written
-// (their threads store to a dummy slot): the buffers are cleared once and those columns stay zero.
-// Rows past the end of the operand come back as zeros from the buffer view.
-template <int KS>
-struct Stager {
-  static constexpr int kGran = 4 * KS;             // 16-byte granules per (zero padded) row
-  static constexpr int kRowBytes = KS * 64 + 32;   // LDS row pitch
-  static constexpr int kTotal = kChunk * kGran;
-  static constexpr int kPer = (kTotal + kThreads - 1) / kThreads;
-  static constexpr int kDummy = kChunk * kRowBytes;  // 16 bytes nobody reads
-  static constexpr int kBytes = kChunk * kRowBytes + 16;
-  u32x4 regs[kPer];
-  uint32_t goff[kPer];   // source byte offset inside a chunk
-  uint32_t loff[kPer];   // LDS byte offset inside a stage buffer (kDummy for padding granules)
+// Global -> LDS staging of the streamed operand, kChunk rows at a time, without passing through
+// registers: buffer loads with the LDS as destination write 16 bytes per lane, 1 KiB per wave and
+// instruction, to consecutive LDS addresses, while every lane chooses which 16 bytes of global memory it
+// fetches.  A ring of stages is filled several chunks ahead of its use, so a load has one or two whole
+// chunk periods to arrive and no wave ever waits for memory in the sweep.
+//
+// LDS layout of a stage: kChunk rows of kPitch bytes, no padding.  The 16-byte granule c of row r sits
+// at granule position c ^ swz(r) of its row: a 16-byte fragment read is served in passes of lanes
+// {0-7, 16-23}, {8-15, 24-31}, .. (eight consecutive rows at two neighbouring granule columns), and the
+// swizzle sends those sixteen granules to sixteen different 16-byte slots modulo 256 bytes, i.e. to all
+// 64 banks once.  Granule columns at or past D/8 (the zero padding up to the MFMA k-step, and up to the
+// pitch) are fetched from an offset past the end of the buffer view, which yields zeros; so do rows
+// past the end of the operand.  Behind the rows a stage has room for 64 floats (the column kernel's lse).
+constexpr uint32_t kPastEnd = 0xfffffff0u;   // never inside a view: rows_view keeps sizes below it
 
-  __device__ __forceinline__ void init(int64_t row_bytes, int dgran, int tid) {
+// Stages of the ring in the two big sweeps: four while two workgroups of them fit a CU's 160 KiB (loads
+// then have two to three chunk periods to arrive), two for the 32 KiB stages of D > 128.
+__host__ __device__ constexpr int ring_stages(int ksteps) { return ksteps <= 4 ? 4 : 2; }
+
+template <int AUX>
+__device__ __forceinline__ void dma16(__amdgpu_buffer_rsrc_t view, uint32_t byte_off, char* lds_wave_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(view, (__attribute__((address_space(3))) void*)lds_wave_base, 16,
+                                           (int)byte_off, 0, 0, AUX);
+}
+__device__ __forceinline__ void dma4(__amdgpu_buffer_rsrc_t view, uint32_t byte_off, char* lds_wave_base) {
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(view, (__attribute__((address_space(3))) void*)lds_wave_base, 4,
+                                           (int)byte_off, 0, 0, 0);
+}
+
+// Waits until at most N of this wave's loads are outstanding and all its LDS reads have returned, then
+// meets the other waves.  After it, what every wave loaded before its N newest loads is visible to
+// all, and no wave is still reading what it read before the barrier, so those stages may be refilled.
+// The empty asm statements keep the compiler from moving LDS accesses across the barrier (there is no
+// fence, which would wait for every outstanding load).
+template <int N>
+__device__ __forceinline__ void ring_sync() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (0 << 8));  // vmcnt(N) lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+template <int KS, int NS = ring_stages(KS)>
+struct Ring {
+  static constexpr int kN = NS;
+  static constexpr int kPitch = KS <= 1 ? 64 : KS == 2 ? 128 : KS <= 4 ? 256 : 512;   // LDS row pitch
+  static constexpr int kRowsPerLoad = 1024 / kPitch;                 // rows one wave-wide load covers
+  static constexpr int kPer = kChunk / (kWaves * kRowsPerLoad);     // loads per wave and chunk
+  static constexpr int kRows = kChunk * kPitch;                      // bytes of rows in a stage
+  static constexpr int kStage = kRows + kChunk * 4;                  // rows + 64 floats
+  static constexpr int kBytes = kN * kStage;
+  static constexpr int kSwz = kPitch < 256 ? kPitch : 256;
+  static __host__ __device__ constexpr int swz(int row) { return 2 * ((row * kSwz / 256) & (kSwz / 32 - 1)); }
+
+  uint32_t voff[kPer];   // source byte offset inside a chunk of the granule this lane fetches, per load
+  uint32_t ko[KS];       // LDS byte offset inside a 16-row group of this lane's fragment, per k-step
+  int wave;              // wave-uniform
+
+  __device__ __forceinline__ void init(int64_t row_bytes, int dgran, int lane, int wave_id) {
+    wave = wave_id;
 #pragma unroll
     for (int i = 0; i < kPer; ++i) {
-      const int g = tid + i * kThreads;
-      const int r = min(g / kGran, kChunk - 1), cg = g % kGran;
-      const bool live = (g < kTotal) && (cg < dgran);
-      goff[i] = (uint32_t)r * (uint32_t)row_bytes + (uint32_t)min(cg, dgran - 1) * 16u;
-      loff[i] = live ? (uint32_t)(r * kRowBytes + cg * 16) : (uint32_t)kDummy;
+      const int byte = (wave * kPer + i) * 1024 + lane * 16;   // where the lane's 16 bytes land in the stage
+      const int row = byte / kPitch;
+      const int c = ((byte % kPitch) / 16) ^ swz(row);         // the granule that belongs there
+      voff[i] = (c < dgran) ? (uint32_t)row * (uint32_t)row_bytes + (uint32_t)c * 16u : kPastEnd;
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const int r = lane & 15, c = 4 * ks + (lane >> 4);
+      ko[ks] = (uint32_t)(r * kPitch + ((c ^ swz(r)) * 16));
     }
   }
-  // Clears `bytes` of LDS (a multiple of 16) when some granule columns are padding.
-  static __device__ __forceinline__ void clear(char* lds, int bytes, int dgran, int tid) {
-    if (dgran < kGran) {
-      const u32x4 zero = {0u, 0u, 0u, 0u};
-      for (int o = tid * 16; o < bytes; o += kThreads * 16) *reinterpret_cast<u32x4*>(lds + o) = zero;
-      __syncthreads();
-    }
-  }
-  // Rows [row0, row0 + kChunk) of an operand of nrows rows starting at base.  No branches.
+  // Rows [row0, row0 + kChunk) of the operand into `stage`; rows at or past `nrows` arrive as zeros
+  // without touching memory.
   template <int AUX = 0>
-  __device__ __forceinline__ void load(const char* base, int64_t row_bytes, int row0, int nrows) {
+  __device__ __forceinline__ void issue(const char* base, int64_t row_bytes, int row0, int nrows, char* stage) const {
     const __amdgpu_buffer_rsrc_t view = rows_view(base, row_bytes, row0, nrows);
 #pragma unroll
-    for (int i = 0; i < kPer; ++i) regs[i] = view_load16<AUX>(view, goff[i]);
-  }
-  __device__ __forceinline__ void store(char* lds) const {
-#pragma unroll
-    for (int i = 0; i < kPer; ++i) *reinterpret_cast<u32x4*>(lds + loff[i]) = regs[i];
+    for (int i = 0; i < kPer; ++i) dma16<AUX>(view, voff[i], stage + (wave * kPer + i) * 1024);
   }
   // Fragment of the 16-row group sg of sub-step `sub` (32 rows) for k-step ks.
-  static __device__ __forceinline__ u32x4 frag(const char* lds, int sub, int sg, int ks, int lane) {
-    return *reinterpret_cast<const u32x4*>(lds + (sub * 32 + sg * 16 + (lane & 15)) * kRowBytes + ks * 64 +
-                                           (lane >> 4) * 16);
+  __device__ __forceinline__ u32x4 frag(const char* stage, int sub, int sg, int ks) const {
+    return *reinterpret_cast<const u32x4*>(stage + (sub * 32 + sg * 16) * kPitch + ko[ks]);
   }
 };
 
@@ -284,10 +314,9 @@ struct Stager {
 // the A operand.  A streamed fragment stays put for NG consecutive MFMAs.  When REFILL, each fragment
 // register is reloaded for the sub-step after this one as soon as its MFMAs are issued, a whole
 // sub-step ahead of its use.
-template <int DT, int KS, int NG, bool RESIDENT_IS_KEYS, bool REFILL>
+template <int DT, int KS, int NG, bool RESIDENT_IS_KEYS, bool REFILL, class RingT>
 __device__ __forceinline__ void mma_groups(f32x4 (&n)[NG][2], u32x4 (&f)[2][KS], const u32x4 (&res)[NG][KS],
-                                           const char* next_lds, int next_sub, int lane) {
-  using St = Stager<KS>;
+                                           const RingT& rg, const char* next_lds, int next_sub) {
   const f32x4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int g = 0; g < NG; ++g) {
@@ -303,80 +332,63 @@ __device__ __forceinline__ void mma_groups(f32x4 (&n)[NG][2], u32x4 (&f)[2][KS],
         if (RESIDENT_IS_KEYS) n[g][sg] = mma<DT>(res[g][ks], f[sg][ks], n[g][sg]);
         else n[g][sg] = mma<DT>(f[sg][ks], res[g][ks], n[g][sg]);
       }
-      if (REFILL) f[sg][ks] = St::frag(next_lds, next_sub, sg, ks, lane);
+      if (REFILL) f[sg][ks] = rg.frag(next_lds, next_sub, sg, ks);
+      // MFMAs and LDS reads keep this order (the refill stays a sub-step ahead of its use instead of
+      // sinking to just before it); vector, transcendental and scalar instructions may move across.
+      __builtin_amdgcn_sched_barrier(0x2 | 0x4 | 0x400);
     }
   }
 }
 
-// Branch-free sweep over chunks [ta, tb) of the streamed operand, none of which needs a mask.
-// Chunk t lives in stage buffer t & 1.  On entry chunk ta has been stored to its buffer (not yet
-// published by a barrier) and the staging registers hold chunk ta+1; on exit the same holds for tb,
-// so the general loops can run before or after.
+// Ring protocol.  advance(t) = ring_sync, then the load of chunk t + kN - 1 into the stage chunk t - 1
+// lived in.  A loop calls it once per chunk, in order, before it first touches chunk t; loads are issued
+// in chunk order, kPer (+1 with an lse row) per wave and chunk, so at that point "all but the newest
+// kN - 2 chunks' loads have arrived" is exactly "chunk t has arrived".  Before the first advance the
+// loads of the first kN - 1 chunks of the sweep have been issued.
 //
+// Branch-free sweep over chunks [ta, tb) of the streamed operand, none of which needs a mask.
 // Steady state, per chunk t (two sub-steps s0, s1), one barrier:
-//     barrier            chunk t+1 published; nobody reads chunk t from LDS any more
-//     MFMA(s1 of t)   || VALU of s0 of t   || fragments <- s0 of t+1   || stage t+2: regs -> LDS,
-//     MFMA(s0 of t+1) || VALU of s1 of t   || fragments <- s1 of t+1   || regs <- chunk t+3
-// Every LDS read is issued a sub-step before its use, every global load a chunk before its store,
-// every LDS store half a chunk before the barrier that publishes it.
-// aux_of(lds, sub) reads what the consumer needs per sub-step besides the scores (the column
+//     advance(t+1)       chunk t+1 visible; nobody reads chunk t any more, its stage is being refilled
+//     MFMA(s1 of t)   || VALU of s0 of t   || fragments <- s0 of t+1
+//     MFMA(s0 of t+1) || VALU of s1 of t   || fragments <- s1 of t+1
+// Every LDS read is issued a sub-step before its use.
+// aux_of(stage, sub) reads what the consumer needs per sub-step besides the scores (the column
 // kernel: lse of the lane's queries); it travels with the fragments so that it too is read before
-// the barrier that lets other waves overwrite the buffer.
-// staging_sweep below is the same sequence of barriers, LDS stores and global loads without the
-// arithmetic, for a wave whose resident rows are all padding.
-template <class StoreF, class LoadF>
-__device__ __forceinline__ void staging_sweep(int ta, int tb, char* smem, int stage_bytes, StoreF&& stage_store,
-                                              LoadF&& stage_load) {
-  if (ta >= tb) return;
-  __syncthreads();
-  stage_store(smem + ((ta + 1) & 1) * stage_bytes);
-  stage_load(ta + 2);
-  for (int t = ta; t + 1 < tb; ++t) {
-    __syncthreads();
-    stage_store(smem + (t & 1) * stage_bytes);
-    stage_load(t + 3);
-  }
-}
-
-template <int DT, int KS, int NG, bool RESIDENT_IS_KEYS, class Aux, class StoreF, class LoadF, class AuxF,
-          class ConsumeF>
-__device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[NG][KS], char* smem,
-                                                int stage_bytes, int lane, StoreF&& stage_store,
-                                                LoadF&& stage_load, AuxF&& aux_of, ConsumeF&& consume) {
-  using St = Stager<KS>;
+// the barrier that lets the stage be refilled.
+template <int DT, int KS, int NG, bool RESIDENT_IS_KEYS, class Aux, class RingT, class AdvF, class StageF,
+          class AuxF, class ConsumeF>
+__device__ __forceinline__ void pipelined_sweep(int ta, int tb, const u32x4 (&res)[NG][KS], const RingT& rg,
+                                                AdvF&& advance, StageF&& stage_of, AuxF&& aux_of,
+                                                ConsumeF&& consume) {
   if (ta >= tb) return;
   u32x4 f[2][KS];
   f32x4 pa[NG][2], pb[NG][2];  // scores of the sub-step being consumed / being produced, swapping roles
   Aux af, ap, an;
-  __syncthreads();
-  stage_store(smem + ((ta + 1) & 1) * stage_bytes);
-  stage_load(ta + 2);
+  advance(ta);
   {
-    const char* lds = smem + (ta & 1) * stage_bytes;
+    const char* lds = stage_of(ta);
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      f[0][ks] = St::frag(lds, 0, 0, ks, lane);
-      f[1][ks] = St::frag(lds, 0, 1, ks, lane);
+      f[0][ks] = rg.frag(lds, 0, 0, ks);
+      f[1][ks] = rg.frag(lds, 0, 1, ks);
     }
     ap = aux_of(lds, 0);
-    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pa, f, res, lds, 1, lane);
+    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pa, f, res, rg, lds, 1);
     af = aux_of(lds, 1);
   }
   for (int t = ta; t + 1 < tb; ++t) {
-    const char* nxt = smem + ((t + 1) & 1) * stage_bytes;
-    __syncthreads();
+    advance(t + 1);
+    const char* nxt = stage_of(t + 1);
     an = af;
-    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pb, f, res, nxt, 0, lane);
+    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pb, f, res, rg, nxt, 0);
     af = aux_of(nxt, 0);
     consume(pa, ap);
-    stage_store(smem + (t & 1) * stage_bytes);
-    stage_load(t + 3);
     ap = af;
-    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pa, f, res, nxt, 1, lane);
+    mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, true>(pa, f, res, rg, nxt, 1);
     af = aux_of(nxt, 1);
     consume(pb, an);
   }
-  mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, false>(pb, f, res, nullptr, 0, lane);
+  mma_groups<DT, KS, NG, RESIDENT_IS_KEYS, false>(pb, f, res, rg, nullptr, 0);
   consume(pa, ap);
   consume(pb, af);
 }
@@ -483,10 +495,10 @@ struct NoAux {};
 // default policy is the faster one.
 template <int DT, int KS, bool CAUSAL, int NB, bool STREAM_ONCE>
 __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
-  using St = Stager<KS>;
+  using Rg = Ring<KS>;
   constexpr int NG = 2 * NB;
   constexpr int kTileRows = kWaves * 32 * NB;
-  __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
+  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes];
   int bh, tile, split;
   map_block_split(p, CAUSAL, bh, tile, split);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -508,6 +520,7 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   const int c_begin = split * per_split;
   const int nchunks = min((kend + kChunk - 1) / kChunk, c_begin + per_split);
   const int t_int = min(nchunks, CAUSAL ? min((tile * kTileRows + p.c + 1) / kChunk, p.N / kChunk) : p.N / kChunk);
+  const int keys_end = min(p.N, nchunks * kChunk);   // nothing is fetched from here on
 
   float mref[NG], l[NG];
   int last[NG];  // last key a lane's query may see, minus the lane's row offset in a group
@@ -519,40 +532,37 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
     last[g] = (CAUSAL ? min(p.N - 1, i + p.c) : p.N - 1) - 4 * (lane >> 4);
   }
 
-  // The first chunk of the streamed operand is requested before the resident one, so that both are
-  // in flight together and the first LDS stage does not wait for the resident fragments.
-  St st;
-  st.init(p.k_sr, p.dgran, tid);
-  auto stage_store = [&](char* lds) { st.store(lds); };
-  auto stage_load = [&](int t) { st.template load<(STREAM_ONCE ? kLoadOnce : 0)>(kb, p.k_sr, t * kChunk, p.N); };
-  stage_load(c_begin);
-  u32x4 qf[NG][KS];
-  load_resident<KS, NG>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
-  St::clear(smem, 2 * St::kBytes, p.dgran, tid);
-  stage_store(smem + (c_begin & 1) * St::kBytes);
-  stage_load(c_begin + 1);
+  Rg rg;
+  rg.init(p.k_sr, p.dgran, lane, wave);
+  auto stage_of = [&](int t) { return smem + ((uint32_t)t % Rg::kN) * Rg::kStage; };
+  auto issue = [&](int t) {
+    rg.template issue<(STREAM_ONCE ? kLoadOnce : 0)>(kb, p.k_sr, t * kChunk, keys_end, stage_of(t));
+  };
+  auto advance = [&](int t) {
+    ring_sync<(Rg::kN - 2) * Rg::kPer>();
+    issue(t + Rg::kN - 1);
+  };
+  // The first chunks of the streamed operand are requested before the resident one, so that all of
+  // them are in flight together.
+#pragma unroll
+  for (int i = 0; i < Rg::kN - 1; ++i) issue(c_begin + i);
 
   // A wave whose rows all lie past M (a ragged last tile, fewer than 128 queries) only helps staging.
   if (q0[0] >= p.M) {
-    staging_sweep(c_begin, t_int, smem, St::kBytes, stage_store, stage_load);
-    for (int t = max(t_int, c_begin); t < nchunks; ++t) {
-      __syncthreads();
-      stage_store(smem + ((t + 1) & 1) * St::kBytes);
-      stage_load(t + 2);
-    }
+    for (int t = c_begin; t < nchunks; ++t) advance(t);
+    ring_sync<0>();
     return;
   }
+  u32x4 qf[NG][KS];
+  load_resident<KS, NG>(qf, qb, p.q_sr, q0, p.M, p.dgran, lane);
 
   pipelined_sweep<DT, KS, NG, false, NoAux>(
-      c_begin, t_int, qf, smem, St::kBytes, lane, stage_store, stage_load,
-      [](const char*, int) { return NoAux{}; },
+      c_begin, t_int, qf, rg, advance, stage_of, [](const char*, int) { return NoAux{}; },
       [&](const f32x4(&a)[NG][2], NoAux) { lse_update_groups<NG>(a, p.scale2, mref, l); });
 
   for (int t = max(t_int, c_begin); t < nchunks; ++t) {
-    __syncthreads();  // chunk t published, the other buffer is free
-    stage_store(smem + ((t + 1) & 1) * St::kBytes);
-    stage_load(t + 2);
-    const char* lds = smem + (t & 1) * St::kBytes;
+    advance(t);
+    const char* lds = stage_of(t);
 #pragma unroll
     for (int sub = 0; sub < kChunk / 32; ++sub) {
       const int key0 = t * kChunk + sub * 32;
@@ -564,8 +574,8 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
         f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          acc[0] = mma<DT>(St::frag(lds, sub, 0, ks, lane), qf[g][ks], acc[0]);
-          acc[1] = mma<DT>(St::frag(lds, sub, 1, ks, lane), qf[g][ks], acc[1]);
+          acc[0] = mma<DT>(rg.frag(lds, sub, 0, ks), qf[g][ks], acc[0]);
+          acc[1] = mma<DT>(rg.frag(lds, sub, 1, ks), qf[g][ks], acc[1]);
         }
         const bool need_mask = (key0 + 32 > p.N) || (CAUSAL && key0 + 31 > qg + p.c);
         if (need_mask) lse_update<true>(acc, p.scale2, mref[g], l[g], last[g] - key0);
@@ -573,6 +583,7 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
       }
     }
   }
+  ring_sync<0>();   // the loads past the last chunk write their zeros before the LDS is given back
 
 #pragma unroll
   for (int g = 0; g < NG; ++g) {
@@ -633,7 +644,7 @@ __host__ __device__ constexpr int col_blocks_per_wave(int ksteps, int mode) {
 // waits for the longest sweep): those launches use 128-key tiles.
 inline int col_tile_blocks(int ksteps, int mode, int N, int64_t bh, bool causal) {
   const int nb = col_blocks_per_wave(ksteps, mode);
-  if (nb == 1) return nb;
+  if (nb != 2) return nb;
   const int64_t wgs2 = bh * ((N + kWaves * 64 - 1) / (kWaves * 64));
   const int cus = chip_cus();
   if (causal) return (wgs2 >= cus && wgs2 <= 2 * cus) ? 1 : 2;
@@ -641,14 +652,13 @@ inline int col_tile_blocks(int ksteps, int mode, int N, int64_t bh, bool causal)
 }
 
 template <int DT, int KS, bool CAUSAL, int MODE, int NB>
-__global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p) {
-  using St = Stager<KS>;
+__global__ __launch_bounds__(kThreads, (NB > 2 ? 1 : 2)) void col_reduce_kernel(const Params p) {
+  using Rg = Ring<KS>;
   constexpr int NG = 2 * NB;
   constexpr int kTileRows = kWaves * 32 * NB;
-  constexpr int kStage = St::kBytes + kChunk * 4;     // rows + their lse
   constexpr int kRed = kWaves * NG * 4 * 64 * 4;      // end-of-sweep transpose buffer
-  constexpr int kSmem = (2 * kStage > kRed) ? 2 * kStage : kRed;
-  __shared__ __attribute__((aligned(16))) char smem[kSmem];
+  constexpr int kSmem = (Rg::kBytes > kRed) ? Rg::kBytes : kRed;
+  __shared__ __attribute__((aligned(1024))) char smem[kSmem];
   int bh, tile;
   map_block(p, false, bh, tile);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -668,55 +678,53 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
     cmax[g] = (f32x4){kNegInf, kNegInf, kNegInf, kNegInf};
   }
 
-  // Query chunks [t0, nchunks) can see keys of this tile.  From chunk t_int on every query sees
-  // all of them: those chunks take the branch-free pipelined sweep (rows past M carry lse = +inf
-  // and add 2^-inf = 0, keys past N are computed and never stored, so neither needs a mask).
+  // Query chunks [t0, nchunks) can see keys of this tile.  Chunks [t_int, nfull) are whole chunks whose
+  // queries all see every key of the tile: they take the branch-free pipelined sweep (keys past N are
+  // computed and never stored, so they need no mask).  The chunks on the causal diagonal before them
+  // and a ragged last chunk (rows past M read as zeros, their lse too) take the general loop.
   const int nchunks = (p.M + kChunk - 1) / kChunk;
   const int t0 = CAUSAL ? max(0, tile * kTileRows - p.c) / kChunk : 0;
-  const int t_int = CAUSAL ? min(nchunks, max(t0, (tile * kTileRows + kTileRows - 1 - p.c + kChunk - 1) / kChunk)) : 0;
+  const int nfull = max(t0, p.M / kChunk);
+  const int t_int = CAUSAL ? min(nfull, max(t0, (tile * kTileRows + kTileRows - 1 - p.c + kChunk - 1) / kChunk)) : 0;
   // lim = i + c - key0(group) - 4*(lane/16), with i the lane's query in group 0 of the current sub-tile
   const int lim_lane = (lane & 15) + p.c - 4 * (lane >> 4);
 
-  // A stage is kChunk query rows plus their lse.  The lse value loaded for chunk t is first
-  // touched when the stage is stored, a chunk after its load was issued.
-  St st;
-  float lse_reg;
-  bool lse_live;
-  st.init(p.q_sr, p.dgran, tid);
-  auto stage_load = [&](int t) {
-    st.load(qb, p.q_sr, t * kChunk, p.M);
-    const int i = t * kChunk + (tid & (kChunk - 1));  // threads 64.. duplicate threads 0..63
-    lse_reg = lse[min(i, p.M - 1)];
-    lse_live = (i < p.M);
+  // A stage is kChunk query rows plus their lse.
+  Rg rg;
+  rg.init(p.q_sr, p.dgran, lane, wave);
+  auto stage_of = [&](int t) { return smem + ((uint32_t)t % Rg::kN) * Rg::kStage; };
+  auto issue = [&](int t) {
+    char* stage = stage_of(t);
+    rg.issue(qb, p.q_sr, t * kChunk, p.M, stage);
+    const __amdgpu_buffer_rsrc_t view = rows_view(reinterpret_cast<const char*>(lse), 4, t * kChunk, p.M);
+    dma4(view, (uint32_t)lane * 4u, stage + Rg::kRows);   // every wave writes the same 64 values: no branch
   };
-  auto stage_store = [&](char* lds) {
-    st.store(lds);
-    // +inf for rows past M: they contribute 2^-inf = 0
-    reinterpret_cast<float*>(lds + St::kBytes)[tid & (kChunk - 1)] = lse_live ? lse_reg : kPosInf;
+  auto advance = [&](int t) {
+    ring_sync<(Rg::kN - 2) * (Rg::kPer + 1)>();
+    issue(t + Rg::kN - 1);
   };
   auto aux_of = [&](const char* lds, int sub) {
-    const float* v = reinterpret_cast<const float*>(lds + St::kBytes) + sub * 32 + (lane & 15);
+    const float* v = reinterpret_cast<const float*>(lds + Rg::kRows) + sub * 32 + (lane & 15);
     return LsePair{{v[0], v[16]}};
   };
-  // The first chunk of the streamed operand is requested before the resident one, so that both are
-  // in flight together and the first LDS stage does not wait for the resident fragments.
-  stage_load(t0);
+  // The first chunks of the streamed operand are requested before the resident one, so that all of
+  // them are in flight together.
+#pragma unroll
+  for (int i = 0; i < Rg::kN - 1; ++i) issue(t0 + i);
   u32x4 kf[NG][KS];
   load_resident<KS, NG>(kf, kb, p.k_sr, k0, p.N, p.dgran, lane);
-  St::clear(smem, 2 * kStage, p.dgran, tid);
-  stage_store(smem + (t0 & 1) * kStage);
-  stage_load(t0 + 1);
 
-  for (int t = t0; t < t_int; ++t) {
-    __syncthreads();  // chunk t published, the other buffer is free
-    stage_store(smem + ((t + 1) & 1) * kStage);
-    stage_load(t + 2);
-    const char* lds = smem + (t & 1) * kStage;
+  auto general_chunk = [&](int t) {
+    advance(t);
+    const char* lds = stage_of(t);
 #pragma unroll
     for (int sub = 0; sub < kChunk / 32; ++sub) {
       const int qs = t * kChunk + sub * 32;  // first query of the sub-tile
       if (qs >= p.M) continue;
-      const LsePair lq = aux_of(lds, sub);
+      LsePair lq = aux_of(lds, sub);
+      // +inf for rows past M: they contribute 2^-inf = 0
+      if (qs + (lane & 15) >= p.M) lq.v[0] = kPosInf;
+      if (qs + 16 + (lane & 15) >= p.M) lq.v[1] = kPosInf;
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
         const int kg = k0[g];
@@ -725,60 +733,71 @@ __global__ __launch_bounds__(kThreads, 2) void col_reduce_kernel(const Params p)
         f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          acc[0] = mma<DT>(kf[g][ks], St::frag(lds, sub, 0, ks, lane), acc[0]);
-          acc[1] = mma<DT>(kf[g][ks], St::frag(lds, sub, 1, ks, lane), acc[1]);
+          acc[0] = mma<DT>(kf[g][ks], rg.frag(lds, sub, 0, ks), acc[0]);
+          acc[1] = mma<DT>(kf[g][ks], rg.frag(lds, sub, 1, ks), acc[1]);
         }
         const bool need_mask = CAUSAL && (kg + 15 > qs + p.c);
         if (need_mask) col_update<true, MODE>(acc, p.scale2, lq.v, csum[g], cmax[g], lim_lane + qs - kg);
         else col_update<false, MODE>(acc, p.scale2, lq.v, csum[g], cmax[g], 0);
       }
     }
-  }
+  };
+
+  for (int t = t0; t < t_int; ++t) general_chunk(t);
 
   pipelined_sweep<DT, KS, NG, true, LsePair>(
-      t_int, nchunks, kf, smem, kStage, lane, stage_store, stage_load, aux_of,
+      t_int, nfull, kf, rg, advance, stage_of, aux_of,
       [&](const f32x4(&a)[NG][2], const LsePair& lq) {
         // the lse values are first touched here, a sub-step after their LDS read was issued
 #pragma unroll
         for (int g = 0; g < NG; ++g) col_update<false, MODE>(a[g], p.scale2, lq.v, csum[g], cmax[g], 0);
       });
 
-  // Reduce over the 16 query lanes: transpose through LDS, one output key per lane.
+  for (int t = nfull; t < nchunks; ++t) general_chunk(t);
+
+  // Reduce over the 16 query lanes: transpose through LDS, one output key per lane and pass; a pass
+  // writes out four of the wave's groups.
   float* red = reinterpret_cast<float*>(smem) + wave * (NG * 4 * 64);
   const int w = lane & 15;                 // key inside its group
-  const int grp = lane >> 4;               // which of the wave's groups this lane writes out
-  const int idx = grp * 4 + (w & 3);
-  const float* src = red + idx * 64 + (w >> 2) * 16;
-  const int key = k0[grp < NG ? grp : 0] + w;
-  const bool active = grp < NG;            // lanes 32.. idle when a wave keeps two groups
-  const bool writer = active && key < p.N;
+  ring_sync<0>();   // every load has landed (those past the last chunk write zeros): the LDS can be reused
   if (MODE != kModeMax) {
-    __syncthreads();
 #pragma unroll
     for (int g = 0; g < NG; ++g)
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[(g * 4 + r) * 64 + lane] = csum[g][r];
     __syncthreads();
-    if (active) {
-      float v = 0.f;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) v += src[(j + lane) & 15];
-      if (writer) p.out[(int64_t)bh * p.N + key] = v;
+    for (int g4 = 0; g4 < NG; g4 += 4) {
+      const int grp = g4 + (lane >> 4);      // which of the wave's groups this lane writes out
+      if (grp < NG) {                        // lanes 32.. idle when a wave keeps two groups
+        const float* src = red + (grp * 4 + (w & 3)) * 64 + (w >> 2) * 16;
+        float v = 0.f;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v += src[(j + lane) & 15];
+        const int key = k0[grp] + w;
+        if (key < p.N) p.out[(int64_t)bh * p.N + key] = v;
+      }
     }
   }
   if (MODE != kModeSum) {
-    __syncthreads();
+    if (MODE == kModeBoth) __syncthreads();
 #pragma unroll
     for (int g = 0; g < NG; ++g)
 #pragma unroll
       for (int r = 0; r < 4; ++r) red[(g * 4 + r) * 64 + lane] = cmax[g][r];
     __syncthreads();
-    if (active) {
-      float v = kNegInf;
 #pragma unroll
-      for (int j = 0; j < 16; ++j) v = fmaxf(v, src[(j + lane) & 15]);
-      float* dst = (MODE == kModeBoth) ? p.out2 : p.out;
-      if (writer) dst[(int64_t)bh * p.N + key] = fast_exp2(v);
+    for (int g4 = 0; g4 < NG; g4 += 4) {
+      const int grp = g4 + (lane >> 4);
+      if (grp < NG) {
+        const float* src = red + (grp * 4 + (w & 3)) * 64 + (w >> 2) * 16;
+        float v = kNegInf;
+#pragma unroll
+        for (int j = 0; j < 16; ++j) v = fmaxf(v, src[(j + lane) & 15]);
+        float* dst = (MODE == kModeBoth) ? p.out2 : p.out;
+        const int key = k0[grp] + w;
+        if (key < p.N) dst[(int64_t)bh * p.N + key] = fast_exp2(v);
+      }
     }
   }
 }
@@ -798,8 +817,8 @@ constexpr int kSmallRows = 128;
 
 template <int DT, int KS, bool CAUSAL, int MODE, int NG>
 __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(const Params p) {
-  using St = Stager<KS>;
-  __shared__ __attribute__((aligned(16))) char smem[2 * St::kBytes];
+  using Rg = Ring<KS, 3>;   // three workgroups share a CU: 3 x 3 stages of 16 KiB
+  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes];
   int bh, split;
   map_group(p, p.splits, bh, split);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -813,29 +832,19 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
   const int per = (nchunks + p.splits - 1) / p.splits;
   const int c0 = split * per, c1 = min(nchunks, c0 + per);
   if (c0 >= c1) return;  // the whole workgroup
+  const int keys_end = min(p.N, c1 * kChunk);   // nothing is fetched from here on
 
-  // Staging registers for two chunks: the loads of chunk t+3 are issued while chunk t is computed and
-  // land two barriers later, so a workgroup keeps two chunks of keys in flight.
-  St st;
-  st.init(p.k_sr, p.dgran, tid);
-  u32x4 ra[St::kPer], rb[St::kPer];
+  // The ring keeps two chunks of keys in flight per workgroup.
+  Rg rg;
+  rg.init(p.k_sr, p.dgran, lane, wave);
   const bool once = p.stream_once != 0;
-  auto load = [&](u32x4(&r)[St::kPer], int t) {
-    const __amdgpu_buffer_rsrc_t view = rows_view(kb, p.k_sr, t * kChunk, p.N);
-    if (once) {
-#pragma unroll
-      for (int i = 0; i < St::kPer; ++i) r[i] = view_load16<kLoadOnce>(view, st.goff[i]);
-    } else {
-#pragma unroll
-      for (int i = 0; i < St::kPer; ++i) r[i] = view_load16(view, st.goff[i]);
-    }
+  auto stage_of = [&](int t) { return smem + ((uint32_t)t % Rg::kN) * Rg::kStage; };
+  auto issue = [&](int t) {
+    if (once) rg.template issue<kLoadOnce>(kb, p.k_sr, t * kChunk, keys_end, stage_of(t));
+    else rg.template issue<0>(kb, p.k_sr, t * kChunk, keys_end, stage_of(t));
   };
-  auto store = [&](const u32x4(&r)[St::kPer], char* lds) {
 #pragma unroll
-    for (int i = 0; i < St::kPer; ++i) *reinterpret_cast<u32x4*>(lds + st.loff[i]) = r[i];
-  };
-  load(ra, c0);
-  load(rb, c0 + 1);
+  for (int i = 0; i < Rg::kN - 1; ++i) issue(c0 + i);
 
   // -lse of the lane's queries; -inf hides the rows past M
   const int qrow = 4 * (lane >> 4);
@@ -853,18 +862,13 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
   }
   u32x4 qf[NG][KS];
   load_resident<KS, NG>(qf, qb, p.q_sr, rows, p.M, p.dgran, lane);
-  St::clear(smem, 2 * St::kBytes, p.dgran, tid);
-  store(ra, smem + (c0 & 1) * St::kBytes);
-  load(ra, c0 + 2);
 
   float* out_sum = p.out + (int64_t)bh * p.N;
   float* out_max = ((MODE == kModeBoth) ? p.out2 : p.out) + (int64_t)bh * p.N;
-  // Chunk t: r holds chunk t+1 and is refilled with chunk t+3.
-  auto step = [&](int t, u32x4(&r)[St::kPer]) {
-    __syncthreads();  // chunk t published, the other buffer is free
-    store(r, smem + ((t + 1) & 1) * St::kBytes);
-    load(r, t + 3);
-    const char* lds = smem + (t & 1) * St::kBytes;
+  for (int t = c0; t < c1; ++t) {
+    ring_sync<(Rg::kN - 2) * Rg::kPer>();   // chunk t visible, the stage of chunk t - 1 is free
+    issue(t + Rg::kN - 1);
+    const char* lds = stage_of(t);
     const int key = t * kChunk + 16 * wave + (lane & 15);
     // query i sees the key iff key <= i + c; chunks that end at or before key c need no mask
     const bool need_mask = CAUSAL && (t * kChunk + kChunk - 1 > p.c);
@@ -878,7 +882,7 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
       for (int g = 0; g < 4; ++g) acc[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const u32x4 kfrag = St::frag(lds, wave >> 1, wave & 1, ks, lane);
+        const u32x4 kfrag = rg.frag(lds, wave >> 1, wave & 1, ks);
 #pragma unroll
         for (int g = 0; g < 4; ++g) acc[g] = mma<DT>(qf[gb + g][ks], kfrag, acc[g]);
       }
@@ -903,11 +907,8 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
       vmax = fmaxf(vmax, __shfl_xor(vmax, 32));
       if (lane < 16 && key < p.N) out_max[key] = fast_exp2(vmax);
     }
-  };
-  for (int t = c0; t < c1; t += 2) {
-    step(t, rb);
-    if (t + 1 < c1) step(t + 1, ra);
   }
+  ring_sync<0>();   // the loads past the last chunk write their zeros before the LDS is given back
 }
 
 // ---------------------------------------------------------------------------------------------
