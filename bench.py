@@ -1,18 +1,25 @@
 #!/usr/bin/env python3
 """Benchmark of the column-reduction hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cpu-heads H]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cpu-heads H] [--no-configs]
 
 One step = one fcr_colreduce call (row-statistics kernel + column-reduce kernel) on the headline
-workload: causal, B=1, H=32, M=N=8192, D=128, fp16, reduction=sum, inputs
-resident in HBM, buffers preallocated.  Prints ONE JSON line.
+workload: causal, B=1, H=32, M=N=8192, D=128, fp16, reduction=sum, inputs resident in HBM, buffers
+preallocated.  Prints ONE JSON line.
 
-value        effective TFLOP/s = (4*B*H*M*N*D / 2) / time per call (flop convention of the metric).
+value        effective TFLOP/s = (4*B*H*M*N*D / 2) / wall time per step over exactly K steps between
+             device synchronisations, after W warm-up steps.  Before the warm-up an untimed conditioning
+             phase (`config.conditioning`) runs the same call for a fixed time so that the GPU has left
+             its idle clocks; it is outside both `warmup` and `steps`.  `ms_per_step_events` times the
+             same K steps with events on the launch stream.
 roofline     the slower of the two kernels, timed alone with events on the launch stream, against
              the dense fp16 MFMA peak; `kernels` lists both.
 cpu_baseline the CPU oracle (fp32 matmul, mask, softmax, column sum; chunked over query rows)
              timed on this host's cores on a sample of heads of the same workload; the same
              sample is used to check the GPU result against the tolerance of the metric.
+configs      the five named workloads of the benchmark set: ms per call (events), TFLOP/s by the
+             metric's convention, fraction of the MFMA (and, for the decode-shaped one, HBM) roofline,
+             the CPU oracle timed on a sample of heads, and the tolerance verdict per reduction.
 """
 from __future__ import annotations
 
@@ -25,20 +32,102 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-PEAK_FP16_DENSE_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/CU/clk, MI355X published dense fp16
+PEAK_FP16_DENSE_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/CU/clk, MI355X published dense fp16 (= bf16)
+PEAK_HBM_TBPS = 8.0
 # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # scaled by the same counters on a 256 MiB device copy (FETCH unit 2 KiB, WRITE unit 1 KiB);
 # the summary of those runs is profiles/headline_causal_8192_fp16.md.
 HBM_TRAFFIC_BYTES = {"row_lse_kernel": 198.1e6 + 1.05e6, "col_reduce_kernel": 186.0e6 + 1.05e6}
+CONDITIONING_SECONDS = 0.4
+
+
+def _events_ms(torch, fn, reps):
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    a.record()
+    for _ in range(reps):
+        fn()
+    b.record()
+    b.synchronize()
+    return a.elapsed_time(b) / reps
+
+
+def _close(torch, got, want, reduction):
+    """Tolerance of the metric: rtol 2e-3 / atol 1e-5 for sum and mean, 2e-3 relative for max."""
+    err = (got - want).abs()
+    if reduction == "max":
+        rel = float((err / want.abs().clamp_min(1e-30)).max())
+        return rel <= 2e-3, rel
+    ok = bool((err <= 1e-5 + 2e-3 * want.abs()).all())
+    return ok, float((err / (1e-5 + 2e-3 * want.abs())).max())   # worst error in units of the tolerance
+
+
+def run_configs(torch, fca, colreduce_ref, inputs, cores):
+    """The five named workloads.  GPU: flash_colreduce (fp32 result) timed with events; CPU: the oracle
+    on a head sample, timed once (configs 4, 5) or best of three (1-3); parity on that sample."""
+    dev = torch.device("cuda:0")
+    specs = [
+        ("config1", inputs.config1, False, ("sum", "mean", "max"), None),
+        ("config2", inputs.config2, False, ("sum", "mean", "max"), None),
+        ("config3", inputs.config3, True, ("sum", "mean", "max"), None),
+        ("config4", inputs.config4, True, ("sum",), [0, 10, 21, 31]),
+        ("config5", inputs.config5, True, ("mean", "max"), [0, 9, 17, 31]),
+    ]
+    out = []
+    for name, make, causal, reductions, heads in specs:
+        q, k = make()
+        b, h, m, d = q.shape
+        n = k.shape[2]
+        qd, kd = q.to(dev), k.to(dev)
+        flop = 4.0 * b * h * m * n * d * (0.5 if causal else 1.0)
+        bytes_alg = b * h * (m + n) * d * q.element_size() + b * h * n * 4
+        hs = list(range(h)) if heads is None else heads
+        qs, ks = q[:, hs].float(), k[:, hs].float()
+        entry = {"name": name, "shape": {"B": b, "H": h, "M": m, "N": n, "D": d}, "dtype": str(q.dtype).split(".")[-1],
+                 "causal": causal, "flop_per_call": flop, "algorithmic_bytes": bytes_alg,
+                 "cpu_heads": len(hs), "cpu_cores": cores, "reductions": {}}
+        for red in reductions:
+            fn = lambda: fca.flash_colreduce(qd, kd, red, is_causal=causal, out_dtype=torch.float32)
+            got = fn()
+            torch.cuda.synchronize()
+            reps = 5 if flop > 2e12 else (20 if flop > 1e11 else 100)
+            for _ in range(max(2, reps // 4)):
+                fn()
+            ms = _events_ms(torch, fn, reps)
+            cpu_s = None
+            for _ in range(1 if flop > 1e11 else 3):
+                t0 = time.perf_counter()
+                want = colreduce_ref(qs, ks, red, causal)
+                dt = time.perf_counter() - t0
+                cpu_s = dt if cpu_s is None else min(cpu_s, dt)
+            ok, worst = _close(torch, got[:, hs].cpu(), want, red)
+            r = {"ms": ms, "tflops": flop / (ms * 1e-3) / 1e12,
+                 "frac_mfma_peak": flop / (ms * 1e-3) / 1e12 / PEAK_FP16_DENSE_TFLOPS,
+                 "cpu_ms_per_call_extrapolated": cpu_s * 1e3 * h / len(hs),
+                 "cpu_tflops": flop * len(hs) / h / cpu_s / 1e12, "pass": ok,
+                 ("max_rel_err" if red == "max" else "worst_err_over_tol"): worst}
+            if name == "config3":
+                # decode shaped: bound by reading K; also the flop count of the scores actually visible
+                visible = sum(min(n, i + max(n - m, 0) + 1) for i in range(m)) / float(m * n)
+                r["tflops_visible_scores"] = 4.0 * b * h * m * n * d * visible / (ms * 1e-3) / 1e12
+                r["frac_hbm_peak"] = bytes_alg / (ms * 1e-3) / 1e12 / PEAK_HBM_TBPS
+            entry["reductions"][red] = r
+        entry["pass"] = all(r["pass"] for r in entry["reductions"].values())
+        out.append(entry)
+        del qd, kd, q, k, qs, ks
+        torch.cuda.empty_cache()
+    return out
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=100)
-    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--cpu-heads", type=int, default=32,
                     help="heads of the workload the CPU oracle is timed on (0 = skip)")
+    ap.add_argument("--no-configs", action="store_true", help="skip the five named workloads")
+    ap.add_argument("--conditioning", type=float, default=CONDITIONING_SECONDS,
+                    help="seconds of untimed calls before the warm-up (0 = none)")
     ap.add_argument("--copy-calib", action="store_true",
                     help="also run one plain 256 MiB device copy, as the known-size reference for "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE counters")
@@ -51,6 +140,7 @@ def main():
         sys.exit(2)
 
     import torch
+    import flash_colreduce_amd as fca
     from flash_colreduce_amd import _lib
     from tests import _inputs
 
@@ -81,27 +171,33 @@ def main():
         _lib.check(lib.fcr_col_reduce(q.data_ptr(), k.data_ptr(), lse.data_ptr(), out.data_ptr(), *common,
                                       _lib.REDUCE_SUM, 1, stream))
 
+    # conditioning: the same call, untimed, until the clocks have left idle
+    cond_calls = 0
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < args.conditioning:
+        for _ in range(20):
+            both()
+        torch.cuda.synchronize()
+        cond_calls += 20
+
     for _ in range(args.warmup):
         both()
     torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
+    e0.record()
     for _ in range(args.steps):
         both()
+    e1.record()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-
-    def event_ms(fn, reps):
-        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        fn()
-        a.record()
-        for _ in range(reps):
-            fn()
-        b.record()
-        b.synchronize()
-        return a.elapsed_time(b) / reps
+    ms_per_step_events = e0.elapsed_time(e1) / args.steps
 
     reps = max(args.steps, 10)
-    k1_ms, k2_ms = event_ms(pass1, reps), event_ms(pass2, reps)
+    pass1()
+    k1_ms = _events_ms(torch, pass1, reps)
+    pass2()
+    k2_ms = _events_ms(torch, pass2, reps)
     if args.copy_calib:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -118,17 +214,18 @@ def main():
     dom = max(kernels, key=lambda n: kernels[n]["ms"])
     roofline = {"bound": "mfma", "kernel": dom, "achieved": kernels[dom]["tflops"],
                 "peak": PEAK_FP16_DENSE_TFLOPS, "unit": "TFLOP/s",
-                "frac": kernels[dom]["tflops"] / PEAK_FP16_DENSE_TFLOPS, "traffic": args.traffic_bytes if args.traffic_bytes is not None else HBM_TRAFFIC_BYTES[dom],
+                "frac": kernels[dom]["tflops"] / PEAK_FP16_DENSE_TFLOPS,
+                "traffic": args.traffic_bytes if args.traffic_bytes is not None else HBM_TRAFFIC_BYTES[dom],
                 "kernels": kernels, "whole_call_frac": value / PEAK_FP16_DENSE_TFLOPS}
 
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
     cpu_baseline = None
     parity = None
+    from oracle.colreduce_oracle import colreduce_ref
     if args.cpu_heads > 0:
-        from oracle.colreduce_oracle import colreduce_ref
         hs = min(args.cpu_heads, H)
-        cores = os.cpu_count() or 1
-        cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-        torch.set_num_threads(cores)
         qs, ks = q_cpu[:, :hs].float(), k_cpu[:, :hs].float()
         colreduce_ref(qs[:, :1], ks[:, :1], "sum", True)  # warm the thread pool
         t0 = time.perf_counter()
@@ -144,16 +241,23 @@ def main():
         ok = bool((err <= 1e-5 + 2e-3 * want.abs()).all())
         parity = {"heads_checked": hs, "rtol": 2e-3, "atol": 1e-5, "pass": ok,
                   "max_abs_err": float(err.max()), "max_rel_err": float((err / want.abs().clamp_min(1e-30)).max())}
+    del q, k, out, lse
+    torch.cuda.empty_cache()
+
+    configs = None if args.no_configs else run_configs(torch, fca, colreduce_ref, _inputs, cores)
 
     line = {
         "metric": "effective TFLOP/s (4*B*H*M*N*D, halved for causal) of flash_colreduce sum, "
                   "causal B1 H32 M=N=8192 d128 fp16",
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": ms_per_step, "ms_per_step_events": ms_per_step_events,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp16", "accumulate": "fp32", "data": "synthetic",
         "config": {"workload": "causal B=1 H=32 M=N=8192 D=128 fp16, reduction=sum, seed 0 N(0,1)",
-                   "flop_per_call": flop_call, "frac_of_fp16_dense_peak": value / PEAK_FP16_DENSE_TFLOPS},
-        "roofline": roofline, "cpu_baseline": cpu_baseline, "parity": parity,
+                   "flop_per_call": flop_call, "frac_of_fp16_dense_peak": value / PEAK_FP16_DENSE_TFLOPS,
+                   "conditioning": f"{cond_calls} untimed calls of the same workload over {args.conditioning} s "
+                                   "before the warm-up (GPU clocks leave idle); not part of warmup or steps"},
+        "roofline": roofline, "cpu_baseline": cpu_baseline, "parity": parity, "configs": configs,
     }
     print(json.dumps(line), flush=True)
 
