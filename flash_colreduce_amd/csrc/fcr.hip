@@ -481,8 +481,11 @@ __device__ __forceinline__ void lse_update_groups(const f32x4 (&a)[NG][2], float
   }
 }
 
+// log2(2^a + 2^b); a NaN in either (a row with a NaN or +inf score) stays a NaN: fmaxf / fminf alone
+// would drop it.
 __device__ __forceinline__ float lse_merge(float a, float b) {
   const float hi = fmaxf(a, b), lo = fminf(a, b);
+  if (a != a || b != b) return a + b;
   if (hi == kNegInf) return kNegInf;
   return hi + fast_log2(1.0f + fast_exp2(lo - hi));
 }
@@ -587,7 +590,7 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
 
 #pragma unroll
   for (int g = 0; g < NG; ++g) {
-    float v = (l[g] > 0.f) ? mref[g] + fast_log2(l[g]) : kNegInf;
+    float v = (l[g] == 0.f) ? kNegInf : mref[g] + fast_log2(l[g]);   // l is positive, zero (no key seen) or NaN
     v = lse_merge(v, __shfl_xor(v, 16));  // the four lane groups hold different keys of the same query
     v = lse_merge(v, __shfl_xor(v, 32));
     const int i = q0[g] + lane;
@@ -602,11 +605,16 @@ __global__ __launch_bounds__(256) void lse_combine_kernel(const float* __restric
   const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (r >= rows) return;
   float m = kNegInf;
-  for (int s = 0; s < splits; ++s) m = fmaxf(m, part[s * rows + r]);
+  bool nan = false;   // fmaxf drops a NaN partial
+  for (int s = 0; s < splits; ++s) {
+    const float v = part[s * rows + r];
+    nan = nan || (v != v);
+    m = fmaxf(m, v);
+  }
   float acc = 0.f;
   if (m > kNegInf)
     for (int s = 0; s < splits; ++s) acc += fast_exp2(part[s * rows + r] - m);
-  lse[r] = (m > kNegInf) ? m + fast_log2(acc) : kNegInf;
+  lse[r] = nan ? __builtin_nanf("") : ((m > kNegInf) ? m + fast_log2(acc) : kNegInf);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -936,80 +944,241 @@ __global__ __launch_bounds__(256) void pack_f32_kernel(const float* __restrict__
 
 // ---------------------------------------------------------------------------------------------
 // Keep-mask of the k largest scores of every row (what a pruning caller does with the reduced
-// columns).  One workgroup per row: an 8-bit-digit radix select over the order-preserving integer
-// image of the floats finds the k-th largest value in four counting passes, a last pass writes the
-// mask; elements equal to the threshold are kept from the lowest index up until k are kept.
+// columns).  One workgroup of 1024 threads per row.  Floats are mapped to integers of the same order and
+// the key T of the k-th largest element is found from the top bits down; keys equal to T are kept from
+// the lowest column up until k are kept.
+//
+// Rows of up to 32768 columns (topk_mask_kernel): thread t owns keys [t*VPT, t*VPT + VPT) in registers
+// (VPT = 8 or 32) and T is built bit by bit: T | bit is accepted when at least k keys are >= it.  A pass
+// is one compare and one add per key, one cross-lane sum, one LDS add per wave and one barrier.
+// Longer rows (topk_mask_long_kernel) are re-read from memory in every pass, so T is found eight bits at
+// a time from a 256-bin histogram in LDS; a wave whose keys all fall into one bin (the usual case for
+// the top digits) adds its count with one atomic.
 __device__ __forceinline__ uint32_t order_key(float x) {
   uint32_t b = __builtin_bit_cast(uint32_t, x);
   if (b == 0x80000000u) b = 0u;  // -0 and +0 are one value
   return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);  // monotone in x for all non-NaN floats
 }
+__device__ __forceinline__ float key_value(uint32_t key) {
+  return __builtin_bit_cast(float, (key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
+}
 
-__global__ __launch_bounds__(256) void topk_mask_kernel(const float* __restrict__ scores, uint8_t* __restrict__ mask,
-                                                        float* __restrict__ threshold, int N, int k) {
-  __shared__ uint32_t hist[256];
-  __shared__ uint32_t sh_prefix, sh_need, sh_ties, sh_running;
-  __shared__ uint32_t wave_eq[4];
+constexpr int kTopkThreads = 1024;
+
+// Sum of v over the 64 lanes, as a wave-uniform value: butterflies inside rows of 16 lanes, then the row
+// totals are passed on to the rows behind and lane 63 holds the total.
+__device__ __forceinline__ uint32_t wave_sum(uint32_t v) {
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0xB1, 0xf, 0xf, true);    // quad_perm [1,0,3,2]
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x4E, 0xf, 0xf, true);    // quad_perm [2,3,0,1]
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x141, 0xf, 0xf, true);   // row_half_mirror
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x140, 0xf, 0xf, true);   // row_mirror: every lane has its row's sum
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x142, 0xa, 0xf, false);  // row_bcast:15 into rows 1 and 3
+  v += (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, 0x143, 0xc, 0xf, false);  // row_bcast:31 into rows 2 and 3
+  return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// Exclusive rank of this thread's first tie among the ties of the row, by column, given that thread t
+// owns a contiguous run of columns and has `mine` ties.
+__device__ __forceinline__ uint32_t ties_before(uint32_t mine, uint32_t* wave_eq, int lane, int wave) {
+  uint32_t incl = mine;   // inclusive scan over the wave
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const uint32_t o = __shfl_up(incl, d);
+    if (lane >= d) incl += o;
+  }
+  if (lane == 63) wave_eq[wave] = incl;
+  __syncthreads();
+  uint32_t before = incl - mine;
+  for (int w = 0; w < wave; ++w) before += wave_eq[w];
+  return before;
+}
+
+template <int VPT>
+__global__ __launch_bounds__(kTopkThreads) void topk_mask_kernel(const float* __restrict__ scores,
+                                                                 uint8_t* __restrict__ mask,
+                                                                 float* __restrict__ threshold, int N, int k) {
+  constexpr int kW = kTopkThreads / 64;
+  __shared__ uint32_t cnt[34];       // one counter per pass: nothing to reset between passes
+  __shared__ uint32_t wave_eq[kW];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* s = scores + (int64_t)blockIdx.x * N;
   uint8_t* m = mask + (int64_t)blockIdx.x * N;
-  uint32_t prefix = 0, decided = 0, need = (uint32_t)min(k, N);
+  const uint32_t kk = (uint32_t)min(max(k, 0), N);
+  const int base = tid * VPT;
+
+  uint32_t u[VPT];
+  // 16-byte loads when every row starts on a 16-byte boundary
+  if ((N & 3) == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0) {
+#pragma unroll
+    for (int i = 0; i < VPT; i += 4) {
+      if (base + i < N) {
+        const f32x4 v = *reinterpret_cast<const f32x4*>(s + base + i);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) u[i + e] = order_key(v[e]);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) u[i + e] = 0u;   // padding: below every candidate (candidates are >= 1)
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) u[i] = (base + i < N) ? order_key(s[base + i]) : 0u;
+  }
+  if (tid < 34) cnt[tid] = 0;
+  __syncthreads();
+
+  // number of this wave's keys that satisfy pred(key), as a wave-uniform value: every lane counts its
+  // own keys, one cross-lane sum per call
+  auto wave_count = [&](auto pred) {
+    uint32_t c = 0;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) c += pred(u[i]) ? 1u : 0u;
+    return wave_sum(c);
+  };
+
+  uint32_t T = 0;
+  for (int b = 31; b >= 0; --b) {
+    const uint32_t cand = T | (1u << b);
+    const uint32_t c = wave_count([&](uint32_t x) { return x >= cand; });
+    if (lane == 0 && c != 0) atomicAdd(&cnt[31 - b], c);
+    __syncthreads();
+    if (cnt[31 - b] >= kk) T = cand;
+  }
+  // T is the key of the k-th largest element (all ones if k == 0: nothing is kept)
+  {
+    const uint32_t na = wave_count([&](uint32_t x) { return x > T; });
+    const uint32_t ne = wave_count([&](uint32_t x) { return x == T; });
+    if (lane == 0) {
+      if (na) atomicAdd(&cnt[32], na);
+      if (ne) atomicAdd(&cnt[33], ne);
+    }
+    __syncthreads();
+  }
+  const uint32_t above = cnt[32], ties = cnt[33];
+  const uint32_t need = (kk > above) ? kk - above : 0u;   // how many of the `ties` keys equal to T are kept
+  if (tid == 0 && threshold) threshold[blockIdx.x] = key_value(T);
+
+  uint32_t before = 0;
+  if (need < ties) {   // uniform over the workgroup: some ties are dropped, rank them by column
+    uint32_t mine = 0;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) mine += (u[i] == T) ? 1u : 0u;
+    before = ties_before(mine, wave_eq, lane, wave);
+  }
+
+  // the mask, VPT bytes per thread
+  const bool keep_all_ties = need >= ties;
+  uint8_t out[VPT];
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const bool eq = u[i] == T;
+    const bool keep = (kk > 0) && ((u[i] > T) || (eq && (keep_all_ties || before < need)));
+    if (eq) ++before;
+    out[i] = keep ? 1 : 0;
+  }
+  if ((N & 7) == 0 && (reinterpret_cast<uintptr_t>(mask) & 7) == 0) {
+#pragma unroll
+    for (int i = 0; i < VPT; i += 8) {
+      if (base + i < N) {
+        uint64_t w = 0;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) w |= (uint64_t)out[i + e] << (8 * e);
+        *reinterpret_cast<uint64_t*>(m + base + i) = w;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+      if (base + i < N) m[base + i] = out[i];
+  }
+}
+
+__global__ __launch_bounds__(kTopkThreads) void topk_mask_long_kernel(const float* __restrict__ scores,
+                                                                      uint8_t* __restrict__ mask,
+                                                                      float* __restrict__ threshold, int N, int k) {
+  constexpr int kW = kTopkThreads / 64;
+  __shared__ uint32_t hist[256];
+  __shared__ uint32_t sh_prefix, sh_need, sh_ties;
+  __shared__ uint32_t wave_eq[kW];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const float* s = scores + (int64_t)blockIdx.x * N;
+  uint8_t* m = mask + (int64_t)blockIdx.x * N;
+  const uint32_t kk = (uint32_t)min(max(k, 0), N);
+  uint32_t prefix = 0, decided = 0, need = kk;
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 24 - 8 * pass;
-    hist[tid] = 0;
+    if (tid < 256) hist[tid] = 0;
     __syncthreads();
-    for (int j = tid; j < N; j += 256) {
-      const uint32_t u = order_key(s[j]);
-      if ((u & decided) == prefix) atomicAdd(&hist[(u >> shift) & 255u], 1u);
-    }
-    __syncthreads();
-    if (tid == 0) {
-      uint32_t above = 0;
-      int d = 255;
-      for (; d > 0; --d) {
-        if (above + hist[d] >= need) break;
-        above += hist[d];
+    for (int j0 = 0; j0 < N; j0 += kTopkThreads) {
+      const int j = j0 + tid;
+      const uint32_t x = (j < N) ? order_key(s[j]) : 0u;
+      const bool live = (j < N) && ((x & decided) == prefix);
+      const uint32_t d = (x >> shift) & 255u;
+      const uint64_t lives = __builtin_amdgcn_ballot_w64(live);
+      if (lives == 0) continue;
+      const uint32_t d0 = __builtin_amdgcn_readlane(d, __builtin_ctzll(lives));
+      if (__builtin_amdgcn_ballot_w64(live && d == d0) == lives) {   // one bin for the whole wave
+        if (lane == 0) atomicAdd(&hist[d0], (uint32_t)__builtin_popcountll(lives));
+      } else if (live) {
+        atomicAdd(&hist[d], 1u);
       }
-      sh_prefix = prefix | ((uint32_t)d << shift);
-      sh_need = need - above;  // how many of the elements with this digit are still wanted
-      sh_ties = hist[d];
     }
     __syncthreads();
-    prefix = sh_prefix;
-    need = sh_need;
+    if (tid < 64) {   // one wave walks the bins from the top: 4 bins per lane, suffix sums across lanes
+      uint32_t h[4], tot = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        h[e] = hist[255 - (lane * 4 + e)];   // lane 0 holds the four largest digits
+        tot += h[e];
+      }
+      uint32_t incl = tot;
+#pragma unroll
+      for (int dd = 1; dd < 64; dd <<= 1) {
+        const uint32_t o = __shfl_up(incl, dd);
+        if (lane >= dd) incl += o;
+      }
+      uint32_t above = incl - tot;    // keys in larger digits than this lane's
+      // the digit where the running count first reaches `need`
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (above < need && above + h[e] >= need) {
+          sh_prefix = prefix | ((uint32_t)(255 - (lane * 4 + e)) << shift);
+          sh_need = need - above;
+          sh_ties = h[e];
+        }
+        above += h[e];
+      }
+    }
+    __syncthreads();
+    if (need > 0) {
+      prefix = sh_prefix;
+      need = sh_need;
+    } else {
+      prefix |= 0xffu << shift;   // k == 0: nothing is kept, any threshold above every key will do
+    }
     decided |= 0xffu << shift;
     __syncthreads();
   }
-  // prefix is now the key of the k-th largest element; `need` of the sh_ties elements equal to it are kept
-  const bool ordered = sh_ties != need;
-  if (tid == 0) {
-    sh_running = 0;
-    if (threshold) {
-      const uint32_t b = (prefix & 0x80000000u) ? (prefix ^ 0x80000000u) : ~prefix;
-      threshold[blockIdx.x] = __builtin_bit_cast(float, b);
-    }
+  // prefix is now the key of the k-th largest element; `need` of the sh_ties keys equal to it are kept
+  const uint32_t T = prefix;
+  const uint32_t ties = (kk > 0) ? sh_ties : 0u;
+  if (tid == 0 && threshold) threshold[blockIdx.x] = key_value(T);
+  const int per = (N + kTopkThreads - 1) / kTopkThreads;   // thread t writes columns [t*per, t*per + per)
+  const int base = tid * per;
+  uint32_t before = 0;
+  if (need < ties) {
+    uint32_t mine = 0;
+    for (int i = 0; i < per; ++i) mine += (base + i < N && order_key(s[base + i]) == T) ? 1u : 0u;
+    before = ties_before(mine, wave_eq, lane, wave);
   }
-  __syncthreads();
-  for (int base = 0; base < N; base += 256) {
-    const int j = base + tid;
-    const uint32_t u = (j < N) ? order_key(s[j]) : 0u;
-    const bool eq = (j < N) && (u == prefix) && (k > 0);
-    bool keep = (j < N) && (u > prefix) && (k > 0);
-    if (!ordered) {
-      keep = keep || eq;
-    } else {  // wave-uniform: rank the ties by index
-      const uint64_t ballot = __builtin_amdgcn_ballot_w64(eq);
-      if (lane == 0) wave_eq[wave] = (uint32_t)__builtin_popcountll(ballot);
-      __syncthreads();
-      uint32_t before = sh_running;
-      for (int w = 0; w < wave; ++w) before += wave_eq[w];
-      before += (uint32_t)__builtin_popcountll(ballot & ((1ull << lane) - 1ull));
-      keep = keep || (eq && before < need);
-      __syncthreads();
-      if (tid == 0) sh_running += wave_eq[0] + wave_eq[1] + wave_eq[2] + wave_eq[3];
-      __syncthreads();
-    }
-    if (j < N) m[j] = keep ? 1 : 0;
+  const bool keep_all_ties = need >= ties;
+  for (int i = 0; i < per; ++i) {
+    const int j = base + i;
+    if (j >= N) break;
+    const uint32_t x = order_key(s[j]);
+    const bool eq = x == T;
+    m[j] = ((kk > 0) && ((x > T) || (eq && (keep_all_ties || before < need)))) ? 1 : 0;
+    if (eq) ++before;
   }
 }
 
@@ -1304,8 +1473,11 @@ int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float
 int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream) {
   if (!scores || !mask) return fail(FCR_E_NULL, "null pointer argument");
   if (rows < 1 || rows > 0x7fffffffll || N < 1) return fail(FCR_E_SHAPE, "rows must be in [1, 2^31) and N >= 1");
-  hipLaunchKernelGGL(topk_mask_kernel, dim3((unsigned)rows), dim3(256), 0, static_cast<hipStream_t>(stream), scores,
-                     mask, threshold, N, k);
+  const dim3 grid((unsigned)rows), block(kTopkThreads);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (N <= 8 * kTopkThreads) hipLaunchKernelGGL(topk_mask_kernel<8>, grid, block, 0, s, scores, mask, threshold, N, k);
+  else if (N <= 32 * kTopkThreads) hipLaunchKernelGGL(topk_mask_kernel<32>, grid, block, 0, s, scores, mask, threshold, N, k);
+  else hipLaunchKernelGGL(topk_mask_long_kernel, grid, block, 0, s, scores, mask, threshold, N, k);
   return launched("topk_mask_kernel");
 }
 

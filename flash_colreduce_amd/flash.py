@@ -256,7 +256,10 @@ def topk_keep_mask(scores: torch.Tensor, k: int, return_threshold: bool = False)
     s = scores.contiguous()
     n = s.shape[-1]
     rows = s.numel() // n if n else 0
-    mask = torch.zeros(s.shape, device=s.device, dtype=torch.bool)
+    if rows > 0 and n > 0:
+        mask = torch.empty(s.shape, device=s.device, dtype=torch.bool)   # the kernel writes every entry
+    else:
+        mask = torch.zeros(s.shape, device=s.device, dtype=torch.bool)
     thr = torch.empty(s.shape[:-1], device=s.device, dtype=torch.float32) if return_threshold else None
     if rows > 0 and n > 0:
         with torch.cuda.device(s.device):

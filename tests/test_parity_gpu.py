@@ -136,12 +136,12 @@ def _full_size(q, k, reductions, oracle_heads, what):
 
 def test_config4_full_size():
     q, k = _inputs.config4()
-    _full_size(q, k, ["sum"], [0, 31], "config4")
+    _full_size(q, k, ["sum"], [0, 10, 21, 31], "config4")
 
 
 def test_config5_full_size():
     q, k = _inputs.config5()
-    _full_size(q, k, ["mean", "max"], [17], "config5")
+    _full_size(q, k, ["mean", "max"], [0, 9, 17, 31], "config5")
 
 
 def test_headline_shape_fp16():
@@ -359,6 +359,43 @@ def test_score_jumps_renormalise(causal):
     run_all(q.half(), k.half(), causal, scale=1.0, what="jumps scale 1")
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_nan_and_inf_inputs(causal):
+    """Non-finite inputs.  A row of scores with a NaN or a +inf (inf - inf in the softmax) is a NaN row:
+    every column it may see gets a NaN sum and mean, as in the materialising reference (naive.py:19-28).
+    Columns hidden from every such row are untouched (the reference's materialised softmax makes the
+    hidden entries of a NaN row NaN as well, naive.py:24-25; its kernel, like this one, never visits
+    them, flash.py:198-207), as are rows and (b,h) pairs without one.  The column maximum follows IEEE
+    maxNum (a NaN operand is dropped, like the Triton max at flash.py:123-124), so 'max' is compared on
+    the columns no NaN row sees."""
+    b, h, m, n, d = 1, 4, 150, 260, 64
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=55)
+    q = q.clone()
+    k = k.clone()
+    q[0, 0, 70, 5] = float("nan")          # head 0: a NaN in query 70
+    q[0, 1, 20, 3] = float("inf")          # head 1: an infinity in query 20 (scores +inf and -inf)
+    k[0, 2, 100, 7] = float("-inf")        # head 2: an infinity in key 100: +inf scores for queries with q[7] < 0
+    c = max(n - m, 0)
+    scores = torch.einsum("bhmd,bhnd->bhmn", q.float(), k.float())
+    vis = (torch.arange(m)[:, None] + c >= torch.arange(n)[None, :]) if causal else torch.ones(m, n, dtype=torch.bool)
+    bad = ((torch.isnan(scores) | (scores == float("inf"))) & vis).any(-1)          # [b, h, m]: NaN rows
+    assert bad[0, 0].sum() == 1 and bad[0, 1].sum() == 1 and bad[0, 2].sum() > 10 and not bad[0, 3].any()
+    nan_cols = (bad[..., None] & vis).any(-2)                                          # [b, h, n]
+    q_clean = torch.where(bad[..., None], torch.zeros_like(q), q)   # a zero row adds nothing to columns it cannot see
+    k_clean = torch.nan_to_num(k, neginf=0.0)
+    qd, kd = q.cuda(), k.cuda()
+    for red in REDUCTIONS:
+        got = fca.flash_colreduce(qd, kd, red, is_causal=causal, out_dtype=torch.float32).cpu()
+        want = colreduce_ref(q_clean, k_clean, red, causal)
+        if red != "max":
+            assert torch.equal(torch.isnan(got), nan_cols), red
+        ok = ~nan_cols
+        ok[0, 2] = False     # head 2: the key with the infinity changes every row that sees it
+        if causal:
+            assert ok[0, 0].any() and ok[0, 1].any()
+        check(got[ok], want[ok], red, f"columns no NaN row sees, causal={causal}")
+
+
 def test_heavy_hitter_columns_small():
     q, k = _inputs.config4(heads=2, n=1024)
     run_all(q, k, True, what="config4-small")
@@ -446,7 +483,8 @@ def test_sum_and_max_from_one_sweep(m, n, d, causal, dtype):
 
 
 @pytest.mark.parametrize("n,k", [(1, 1), (5, 2), (256, 100), (257, 256), (1000, 0), (1000, 1000), (1000, 1500),
-                                 (4099, 1024), (32768, 8192)])
+                                 (4099, 1024), (8192, 2048), (8200, 8199), (32768, 8192), (32769, 1), (40000, 5000),
+                                 (70001, 0), (70001, 69000), (131072, 200)])
 def test_topk_keep_mask(n, k):
     from oracle.colreduce_oracle import topk_mask_ref
     g = torch.Generator().manual_seed(n + k)
