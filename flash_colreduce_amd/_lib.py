@@ -14,7 +14,7 @@ import torch  # noqa: F401  (loads the HIP runtime the library binds to)
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfcr.so")
 
-DTYPE_F16, DTYPE_BF16 = 0, 1
+DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 REDUCE_SUM, REDUCE_MAX = 0, 1
 
 _I64x4 = ctypes.c_int64 * 4

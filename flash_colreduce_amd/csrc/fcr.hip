@@ -38,7 +38,7 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int kWaves = 4;
 constexpr int kThreads = kWaves * 64;
-// k-steps are 32 elements of D.  A wave keeps resident rows in groups of 16 (one MFMA operand each);
+// k-steps are 64 bytes of a row: 32 16-bit elements of D, or 16 floats.  A wave keeps resident rows in groups of 16 (one MFMA operand each);
 // two 32-row blocks (four groups) while their fragments fit the register file next to the
 // accumulators (D <= 128: 4 k-steps), one block for larger D.  A workgroup keeps 4 * 32 * blocks rows.
 __host__ __device__ constexpr int blocks_per_wave(int ksteps) { return ksteps <= 4 ? 2 : 1; }
@@ -121,9 +121,19 @@ __device__ __forceinline__ f32x4 mma(u32x4 a, u32x4 b, f32x4 c) {
   if constexpr (DT == FCR_DTYPE_F16) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c,
                                                   0, 0, 0);
-  } else {
+  } else if constexpr (DT == FCR_DTYPE_BF16) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b),
                                                    c, 0, 0, 0);
+  } else {
+    // fp32 operands: the same 16 bytes per lane are four floats, d = 4*(l/16) + e of a 16-float k-step.
+    // v_mfma_f32_16x16x4_f32 number e contracts over the four lane groups' element e, so the four of
+    // them cover the 16 floats once (the order of the terms of a dot product is free).
+    const f32x4 af = __builtin_bit_cast(f32x4, a), bf = __builtin_bit_cast(f32x4, b);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[0], bf[0], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[1], bf[1], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[2], bf[2], c, 0, 0, 0);
+    c = __builtin_amdgcn_mfma_f32_16x16x4f32(af[3], bf[3], c, 0, 0, 0);
+    return c;
   }
 }
 
@@ -1190,16 +1200,20 @@ int fail(int code, const char* what) {
   return code;
 }
 
-int check_strides(const void* ptr, const int64_t s[4], const char* name, int rows, int D) {
+inline int elem_bytes(int dtype) { return dtype == FCR_DTYPE_F32 ? 4 : 2; }
+inline int ksteps_of(int dtype, int D) { return (D * elem_bytes(dtype) + 63) / 64; }
+
+int check_strides(const void* ptr, const int64_t s[4], const char* name, int rows, int D, int esize) {
   if (s[3] != 1) {
     snprintf(g_err, sizeof(g_err), "%s: stride of the last dimension must be 1 (got %lld)", name, (long long)s[3]);
     return FCR_E_STRIDE;
   }
-  if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0 || s[0] % 8 != 0 || s[1] % 8 != 0 || s[2] % 8 != 0 ||
-      s[0] < 0 || s[1] < 0 || s[2] < 0 || s[2] >= (1 << 24)) {
+  const int al = 16 / esize;   // elements per 16 bytes
+  if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0 || s[0] % al != 0 || s[1] % al != 0 || s[2] % al != 0 ||
+      s[0] < 0 || s[1] < 0 || s[2] < 0 || s[2] * esize >= (1 << 25)) {
     snprintf(g_err, sizeof(g_err),
-             "%s: base pointer must be 16-byte aligned, batch/head/row strides non-negative multiples of 8 elements, row stride < 2^24",
-             name);
+             "%s: base pointer must be 16-byte aligned, batch/head/row strides non-negative multiples of 16 bytes (%d elements), row stride < 2^25 bytes",
+             name, al);
     return FCR_E_STRIDE;
   }
   // Rows that overlap (an expanded operand has row stride 0) cannot be described by the buffer views
@@ -1229,26 +1243,31 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
                 const int64_t qs[4], const int64_t ks[4], float scale, bool by_keys, bool causal,
                 int col_mode = kModeSum) {
   if (!q || !k || !qs || !ks) return fail(FCR_E_NULL, "null pointer argument");
-  if (dtype != FCR_DTYPE_F16 && dtype != FCR_DTYPE_BF16) return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16 or FCR_DTYPE_BF16");
+  if (dtype != FCR_DTYPE_F16 && dtype != FCR_DTYPE_BF16 && dtype != FCR_DTYPE_F32)
+    return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16, FCR_DTYPE_BF16 or FCR_DTYPE_F32");
   if (B < 1 || H < 1 || M < 1 || N < 1) return fail(FCR_E_SHAPE, "B, H, M, N must be >= 1");
-  if (D < 8 || D > 32 * kMaxKSteps || D % 8 != 0) return fail(FCR_E_SHAPE, "D must be a multiple of 8 in [8, 256]");
+  const int esize = elem_bytes(dtype);
+  if (D < 1 || D > 64 * kMaxKSteps / esize || (D * esize) % 16 != 0)
+    return fail(FCR_E_SHAPE, esize == 2 ? "D must be a multiple of 8 in [8, 256]"
+                                         : "D must be a multiple of 4 in [4, 128] for FCR_DTYPE_F32");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
   if (bh * (((int64_t)(by_keys ? N : M) + 127) / 128) > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
   if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
-  int rc = check_strides(q, qs, "q", M, D);
+  int rc = check_strides(q, qs, "q", M, D, esize);
   if (rc) return rc;
-  rc = check_strides(k, ks, "k", N, D);
+  rc = check_strides(k, ks, "k", N, D, esize);
   if (rc) return rc;
   // the device is first asked (for its CU count) here, after every argument check
-  const int trows = by_keys ? kWaves * 32 * col_tile_blocks((D + 31) / 32, col_mode, N, bh, causal) : row_tile_rows((D + 31) / 32, M, bh, causal);
+  const int ksteps = ksteps_of(dtype, D);
+  const int trows = by_keys ? kWaves * 32 * col_tile_blocks(ksteps, col_mode, N, bh, causal) : row_tile_rows(ksteps, M, bh, causal);
   const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
   p.q = static_cast<const char*>(q);
   p.k = static_cast<const char*>(k);
-  p.q_sb = qs[0] * 2; p.q_sh = qs[1] * 2; p.q_sr = qs[2] * 2;
-  p.k_sb = ks[0] * 2; p.k_sh = ks[1] * 2; p.k_sr = ks[2] * 2;
+  p.q_sb = qs[0] * esize; p.q_sh = qs[1] * esize; p.q_sr = qs[2] * esize;
+  p.k_sb = ks[0] * esize; p.k_sh = ks[1] * esize; p.k_sr = ks[2] * esize;
   p.H = H; p.M = M; p.N = N;
-  p.dgran = D / 8;
+  p.dgran = D * esize / 16;
   p.c = N > M ? N - M : 0;
   p.scale2 = (float)((double)scale * 1.4426950408889634);
   p.tiles = (int)tiles;
@@ -1266,8 +1285,8 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
 // Key ranges per row tile in the row kernel.  One sweep per workgroup when there is at least one
 // workgroup per CU; otherwise the keys of a tile are split so that about two per CU run, each
 // keeping at least four 64-key chunks.
-int row_splits(int B, int H, int M, int N, int D) {
-  const int trows = row_tile_rows((D + 31) / 32, M, (int64_t)B * H, false);  // same with the mask when wgs < 256
+int row_splits(int B, int H, int M, int N, int ksteps) {
+  const int trows = row_tile_rows(ksteps, M, (int64_t)B * H, false);  // same with the mask when wgs < 256
   const int64_t wgs = (int64_t)B * H * ((M + trows - 1) / trows);
   const int64_t chunks = (N + kChunk - 1) / kChunk;
   const int cus = chip_cus();
@@ -1375,7 +1394,13 @@ const char* fcr_last_error(void) { return g_err; }
 
 size_t fcr_lse_bytes(int B, int H, int M, int N, int D) {
   if (B < 1 || H < 1 || M < 1 || N < 1 || D < 1) return 0;
-  const int splits = row_splits(B, H, M, N, D);
+  // the most any row width asks for (the tile height, hence the split count, depends a little on the
+  // number of 64-byte k-steps of a row), so the size holds for every dtype and D
+  int splits = 1;
+  for (int ks = 1; ks <= kMaxKSteps; ++ks) {
+    const int s = row_splits(B, H, M, N, ks);
+    if (s > splits) splits = s;
+  }
   const size_t rows = (size_t)B * (size_t)H * (size_t)M;
   return rows * sizeof(float) * (splits > 1 ? 1 + (size_t)splits : 1);
 }
@@ -1388,15 +1413,16 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
   int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, false, causal != 0);
   if (rc) return rc;
   p.lse = lse;
-  p.splits = row_splits(B, H, M, N, D);
+  p.splits = row_splits(B, H, M, N, ksteps_of(dtype, D));
   p.part = lse + (int64_t)B * H * M;  // only touched when splits > 1 (see fcr_lse_bytes)
   p.total *= p.splits;
   p.group = head_group(p.bh_count, (int64_t)p.tiles * p.splits, causal != 0);
-  const int ksteps = (D + 31) / 32;
+  const int ksteps = ksteps_of(dtype, D);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal != 0, s)
   if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_LSE) }
-  else { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_LSE) }
+  else if (dtype == FCR_DTYPE_BF16) { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_LSE) }
+  else { FCR_DISPATCH_KS(FCR_DTYPE_F32, ksteps, FCR_CALL_LSE) }
 #undef FCR_CALL_LSE
   rc = launched("row_lse_kernel");
   if (rc || p.splits == 1) return rc;
@@ -1418,9 +1444,10 @@ int col_reduce_any(const void* q, const void* k, const float* lse, float* out, f
   p.lse = const_cast<float*>(lse);
   p.out = out;
   p.out2 = out2;
-  const int ksteps = (D + 31) / 32;
+  const int ksteps = ksteps_of(dtype, D);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  if (M <= kSmallRows && ksteps <= 4) {
+  // (fp32 operands always take the general sweep: they are bound by the fp32 matrix rate, not by reading K)
+  if (M <= kSmallRows && ksteps <= 4 && dtype != FCR_DTYPE_F32) {
     // Few queries: the sweep with all of them resident in every wave and the keys streamed, if the
     // problem fills the chip that way: 512 to 1024 workgroups (at least two per CU), each sweeping at
     // least 16 chunks of keys, or 8 if that is what it takes.
@@ -1448,7 +1475,8 @@ int col_reduce_any(const void* q, const void* k, const float* lse, float* out, f
   }
 #define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal != 0, mode, s)
   if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_COL) }
-  else { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL) }
+  else if (dtype == FCR_DTYPE_BF16) { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL) }
+  else { FCR_DISPATCH_KS(FCR_DTYPE_F32, ksteps, FCR_CALL_COL) }
 #undef FCR_CALL_COL
   return launched("col_reduce_kernel");
 }

@@ -15,7 +15,8 @@ from . import _lib
 
 __all__ = ["flash_colreduce", "flash_colreduce_multi", "row_lse2", "topk_keep_mask"]
 
-_DTYPES = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}
+_DTYPES = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_F32}
+_MAX_ROW_BYTES = 512   # a row the kernels can hold: D <= 256 for 16-bit elements, <= 128 for fp32
 
 
 def _validate(query: torch.Tensor, key: torch.Tensor, reduction: Optional[str]):
@@ -29,7 +30,7 @@ def _validate(query: torch.Tensor, key: torch.Tensor, reduction: Optional[str]):
         )
     if reduction is not None and reduction not in ("sum", "mean", "max"):
         raise ValueError(f"Invalid reduction: {reduction}. Must be 'sum', 'mean', or 'max'.")
-    if query.dtype != key.dtype or (query.dtype not in _DTYPES and query.dtype != torch.float32):
+    if query.dtype != key.dtype or query.dtype not in _DTYPES:
         raise ValueError(
             f"Query and key tensors must both be float16, bfloat16 or float32. "
             f"Got query dtype: {query.dtype}, key dtype: {key.dtype}."
@@ -41,17 +42,19 @@ def _validate(query: torch.Tensor, key: torch.Tensor, reduction: Optional[str]):
 
 
 def _device_layout(x: torch.Tensor) -> torch.Tensor:
-    """What the C ABI needs: unit d stride, 16-byte aligned rows, D a multiple of 8.
+    """What the C ABI needs: unit d stride, 16-byte aligned rows, rows a multiple of 16 bytes.
 
     The reference pads D to a power of two (flash.py:368-373); zero columns do not change <q,k>.
-    Here a copy is made only for D % 8 != 0 or for layouts the kernels cannot address.
+    Here a copy is made only when a row is not a multiple of 16 bytes or for layouts the kernels
+    cannot address.
     """
     d = x.shape[3]
-    if d % 8 != 0:
-        return torch.nn.functional.pad(x, (0, 8 - d % 8))  # new contiguous tensor
+    al = 16 // x.element_size()   # elements per 16 bytes: 8 (fp16, bf16) or 4 (fp32)
+    if d % al != 0:
+        return torch.nn.functional.pad(x, (0, al - d % al))  # new contiguous tensor
     ok = (x.stride(3) == 1 and x.data_ptr() % 16 == 0 and
-          all(x.stride(i) % 8 == 0 and x.stride(i) >= 0 for i in (0, 1, 2)) and
-          x.stride(2) < (1 << 24) and
+          all(x.stride(i) % al == 0 and x.stride(i) >= 0 for i in (0, 1, 2)) and
+          x.stride(2) * x.element_size() < (1 << 25) and
           (x.shape[2] <= 1 or x.stride(2) >= d))  # rows must not overlap (expand() gives stride 0)
     if ok:
         return x
@@ -60,11 +63,11 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
 
 
 def _pack_f32(x: torch.Tensor, is_key: bool) -> torch.Tensor:
-    """fp32 operand -> the fp16 layout the kernels take (see fcr_pack_f32 in include/fcr.h).
-
-    Three fp16 segments [hi|hi|lo] / [hi|lo|hi] when they fit in 256 columns (D <= 80): the product
-    is then good to about 2^-22.  Larger D is rounded to fp16 once, which is what the reference's
-    tl.dot does to fp32 operands on its hardware (TF32 has fewer mantissa bits than fp16)."""
+    """fp32 operand with D > 128 -> fp16 (see fcr_pack_f32 in include/fcr.h): rows of more than 512
+    bytes do not fit the kernels' resident operand, so these are rounded to fp16 once, which keeps one
+    more mantissa bit than the TF32 rounding the reference's tl.dot applies to fp32 operands
+    (flash.py:59,108) but not fp32's range: values beyond +-65504 overflow.  fp32 with D <= 128 never
+    comes here: it is multiplied in fp32."""
     b, h, r, d = x.shape
     dpad = (d + 7) // 8 * 8
     terms = 3 if 3 * dpad <= 256 else 1
@@ -86,7 +89,7 @@ def _launch(query, key, kinds, is_causal, scale):
     n = key.shape[2]
     if scale is None:
         scale = 1 / math.sqrt(d)  # the unpadded D (flash.py:366-367)
-    if query.dtype == torch.float32:
+    if query.dtype == torch.float32 and (d + 3) // 4 * 16 > _MAX_ROW_BYTES:
         q, k = _pack_f32(query, False), _pack_f32(key, True)
     else:
         q = _device_layout(query)
@@ -104,8 +107,7 @@ def _launch(query, key, kinds, is_causal, scale):
     else:
         with torch.cuda.device(dev):
             stream = torch.cuda.current_stream(dev).cuda_stream
-            common = (_lib.DTYPE_F16 if q.dtype == torch.float16 else _lib.DTYPE_BF16,
-                      b, h, m, n, q.shape[3], _lib.strides4(q.stride()), _lib.strides4(k.stride()),
+            common = (_DTYPES[q.dtype], b, h, m, n, q.shape[3], _lib.strides4(q.stride()), _lib.strides4(k.stride()),
                       float(scale))
             causal = int(bool(is_causal))
             if len(kinds) == 1:
@@ -166,7 +168,8 @@ def flash_colreduce(
     """Per-key sum / mean / max over queries of softmax(Q K^T * scale), shape (B, H, N).
 
     Args follow the reference (flash.py:311-352): query (B,H,M,D), key (B,H,N,D), fp16, bf16 or
-    fp32 on the GPU, D <= 256; `is_causal` applies the right-aligned mask (key j visible to query i iff
+    fp32 on the GPU, D <= 256 (fp32 operands are multiplied in fp32 for D <= 128 and rounded to fp16
+    once above that); `is_causal` applies the right-aligned mask (key j visible to query i iff
     j <= i + max(N-M, 0)); `scale` defaults to 1/sqrt(D).
 
     `out_dtype` (keyword only, not in the reference) selects the result dtype.  None reproduces

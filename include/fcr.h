@@ -9,11 +9,14 @@
  * Conventions
  *   - All pointers are DEVICE pointers on the current HIP device.  The library never
  *     allocates, frees or keeps them.
- *   - q is [B,H,M,D], k is [B,H,N,D], 16-bit elements (dtype below).  Strides are in ELEMENTS,
- *     order (batch, head, row, d); the d stride must be 1, row/head/batch strides must be
- *     multiples of 8 elements and the base pointers 16-byte aligned, D a multiple of 8 and
- *     8 <= D <= 256.  (The reference takes any strides, flash.py:292-299; a caller with other
- *     layouts makes a contiguous, zero-padded copy first -- the Python host does.)
+ *   - q is [B,H,M,D], k is [B,H,N,D], fp16, bf16 or fp32 elements (dtype below).  Strides are in
+ *     ELEMENTS, order (batch, head, row, d); the d stride must be 1, row/head/batch strides must be
+ *     multiples of 16 bytes (8 16-bit elements, 4 floats) and the base pointers 16-byte aligned; a row
+ *     must be a multiple of 16 bytes and at most 512 bytes long: D a multiple of 8 in [8, 256] for
+ *     16-bit elements, a multiple of 4 in [4, 128] for fp32.  Rows must not overlap (row stride >= D).
+ *     (The reference takes any strides, flash.py:292-299; a caller with other layouts makes a
+ *     contiguous, zero-padded copy first -- the Python host does.)  fp32 operands are multiplied at
+ *     full precision and range (the reference's tl.dot rounds them to TF32, flash.py:59,108).
  *   - lse is fp32 [B*H, M] contiguous: per query row, log2(sum_j 2^(scale*log2(e)*<q_i,k_j>))
  *     over the keys the row may see.  It is the hand-over between the two kernels.  The buffer
  *     fcr_row_lse / fcr_colreduce write it to must be fcr_lse_bytes(B,H,M,N,D) long (scratch follows
@@ -44,6 +47,7 @@ extern "C" {
 /* element type of q and k */
 #define FCR_DTYPE_F16 0
 #define FCR_DTYPE_BF16 1
+#define FCR_DTYPE_F32 2 /* fp32 operands on the fp32 matrix instructions: D a multiple of 4, at most 128 */
 
 /* column reduction over query rows */
 #define FCR_REDUCE_SUM 0 /* also the numerator of 'mean' (flash.py:121-122) */
@@ -52,7 +56,7 @@ extern "C" {
 /* argument errors */
 #define FCR_E_NULL -1      /* a required pointer is NULL */
 #define FCR_E_DTYPE -2     /* dtype is not FCR_DTYPE_* */
-#define FCR_E_SHAPE -3     /* B,H,M,N < 1, D outside [8,256] or not a multiple of 8, sizes overflow */
+#define FCR_E_SHAPE -3     /* B,H,M,N < 1, a row of D elements not a multiple of 16 bytes in [16,512], sizes overflow */
 #define FCR_E_STRIDE -4    /* d stride != 1 or a stride / base pointer breaks 16-byte alignment */
 #define FCR_E_REDUCTION -5 /* reduction is not FCR_REDUCE_* */
 #define FCR_E_SCALE -6     /* scale is not finite */
@@ -68,9 +72,10 @@ int fcr_version(void);
 const char* fcr_last_error(void);
 
 /*
- * Bytes the lse buffer of fcr_row_lse / fcr_colreduce must have for a problem.  The first
- * B*H*M floats are the result; for few query rows and many keys the row kernel splits the keys of a
- * tile over several workgroups and keeps their partial results behind it.  0 for an empty problem.
+ * Bytes the lse buffer of fcr_row_lse / fcr_colreduce must have for a problem, whatever its dtype and
+ * D.  The first B*H*M floats are the result; for few query rows and many keys the row kernel splits the
+ * keys of a tile over several workgroups and keeps their partial results behind it.  0 for an empty
+ * problem.
  */
 size_t fcr_lse_bytes(int B, int H, int M, int N, int D);
 
@@ -113,7 +118,8 @@ int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float
 int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream);
 
 /*
- * fp32 operands: packs a contiguous fp32 [rows, D] into the fp16 [rows, terms * Dp] (Dp = D rounded up
+ * fp32 operands with D > 128, or as a faster and less exact alternative to FCR_DTYPE_F32 (values must
+ * fit fp16): packs a contiguous fp32 [rows, D] into the fp16 [rows, terms * Dp] (Dp = D rounded up
  * to 8, zero padded) that the kernels above take with D' = terms * Dp and dtype FCR_DTYPE_F16.
  * terms = 3 writes [hi | hi | lo] for queries (is_key = 0) and [hi | lo | hi] for keys (is_key != 0),
  * hi = fp16(x), lo = fp16(x - hi): the kernels then see q.k to about 2^-22.  terms = 1 writes [hi].
