@@ -1,6 +1,7 @@
 """Latency / peak-memory sweep over the reference's 20 benchmark shapes.
 
     python -m flash_colreduce_amd.benchmark [--budget SECONDS] [--no-naive] [--rows 0,13] [--out FILE]
+    python -m flash_colreduce_amd.benchmark --topk
 
 Same shapes and method as the reference's harness (benchmarks/run.py:11-92): fp16, H = 32, D = 128,
 reduction = "sum"; per implementation one call, a 10-call calibration, then `iters` warm-up calls and
@@ -17,6 +18,7 @@ import time
 import torch
 
 from . import flash_colreduce, naive_colreduce
+from .flash import topk_keep_mask
 
 CONFIGS = (
     [dict(b=b, h=32, m=1024, n=1024, d=128, is_causal=False) for b in (1, 4, 16, 64, 256)]
@@ -92,15 +94,54 @@ def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None)
     return rows
 
 
+TOPK_SHAPES = ((32, 8192, 2048), (32, 8192, 64), (32, 32768, 8192), (32, 32768, 512), (256, 8192, 2048),
+               (32, 262144, 65536))
+
+
+def run_topk(out=sys.stdout):
+    """The step a pruning caller takes on the reduced columns: keep-mask of the k largest of every row,
+    against torch.topk (+ the scatter that turns its indices into a mask) on the same GPU.  Times are
+    events around 50 calls after 10 warm-up calls, host overhead of the call included."""
+    def timed(fn):
+        for _ in range(10):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(50):
+            fn()
+        b.record()
+        b.synchronize()
+        return a.elapsed_time(b) / 50 * 1e3
+
+    print(f"{'rows x columns, k':<28} {'topk_keep_mask us':>18} {'torch.topk us':>14} {'topk+scatter us':>16}", file=out)
+    g = torch.Generator(device="cuda").manual_seed(0)
+    for rows, n, k in TOPK_SHAPES:
+        s = torch.rand(rows, n, device="cuda", generator=g)
+
+        def via_torch():
+            idx = torch.topk(s, k, dim=-1).indices
+            return torch.zeros_like(s, dtype=torch.bool).scatter_(1, idx, True)
+
+        t_ours = timed(lambda: topk_keep_mask(s, k))
+        t_topk = timed(lambda: torch.topk(s, k, dim=-1))
+        t_mask = timed(via_torch)
+        assert torch.equal(topk_keep_mask(s, k), via_torch())   # distinct values: both masks are the same set
+        print(f"[{rows}, {n}], k={k:<12} {t_ours:>18.1f} {t_topk:>14.1f} {t_mask:>16.1f}", file=out, flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--budget", type=float, default=2.0, help="seconds of timed calls per implementation")
     ap.add_argument("--no-naive", action="store_true", help="skip the materialising implementation")
     ap.add_argument("--rows", default=None, help="comma separated indices (0..19) of the shapes to run; default all")
     ap.add_argument("--out", default=None, help="also write the table to this file")
+    ap.add_argument("--topk", action="store_true", help="time the top-k keep-mask against torch.topk instead")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("benchmark needs a GPU")
+    if args.topk:
+        run_topk()
+        return
     only = None if args.rows is None else {int(r) for r in args.rows.split(",")}
     if args.out:
         with open(args.out, "w") as f:

@@ -274,6 +274,15 @@ __device__ __forceinline__ void ring_sync() {
   asm volatile("" ::: "memory");
 }
 
+// clamp(x, 0, kChunk) on the scalar unit (written out because the compiler turns min(max()) into a
+// three-operand median that only the vector unit has, which would make everything derived from it,
+// here a buffer descriptor, a per-lane value)
+__device__ __forceinline__ int rows_in_chunk(int rows_left) {
+  int live;
+  asm("s_max_i32 %0, %1, 0\n\ts_min_i32 %0, %0, %2" : "=s"(live) : "s"(rows_left), "n"(kChunk) : "scc");
+  return live;
+}
+
 template <int KS, int NS = ring_stages(KS)>
 struct Ring {
   static constexpr int kN = NS;
@@ -305,13 +314,28 @@ struct Ring {
       ko[ks] = (uint32_t)(r * kPitch + ((c ^ swz(r)) * 16));
     }
   }
-  // Rows [row0, row0 + kChunk) of the operand into `stage`; rows at or past `nrows` arrive as zeros
+  // Chunks are fetched in order, so where the next one comes from is kept as a running address and a
+  // count of the rows left (scalar registers, a handful of scalar instructions per chunk): rows
+  // [row0, nrows) of the operand at `base` are what may be fetched, the rest arrives as zeros
   // without touching memory.
+  const char* next_ptr;
+  int rows_left;
+  uint32_t row_bytes32;
+  __device__ __forceinline__ void start(const char* base, int64_t row_bytes, int row0, int nrows) {
+    next_ptr = base + (int64_t)row0 * row_bytes;
+    rows_left = nrows - row0;
+    row_bytes32 = (uint32_t)row_bytes;
+  }
+  // The next kChunk rows into `stage`.
   template <int AUX = 0>
-  __device__ __forceinline__ void issue(const char* base, int64_t row_bytes, int row0, int nrows, char* stage) const {
-    const __amdgpu_buffer_rsrc_t view = rows_view(base, row_bytes, row0, nrows);
+  __device__ __forceinline__ void issue_next(char* stage) {
+    const int live = rows_in_chunk(rows_left);   // the view covers this chunk's rows only
+    const __amdgpu_buffer_rsrc_t view = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(next_ptr), 0, (int)((uint32_t)live * row_bytes32), 0x00020000);
 #pragma unroll
     for (int i = 0; i < kPer; ++i) dma16<AUX>(view, voff[i], stage + (wave * kPer + i) * 1024);
+    next_ptr += (int64_t)kChunk * row_bytes32;
+    rows_left -= kChunk;
   }
   // Fragment of the 16-row group sg of sub-step `sub` (32 rows) for k-step ks.
   __device__ __forceinline__ u32x4 frag(const char* stage, int sub, int sg, int ks) const {
@@ -350,8 +374,8 @@ __device__ __forceinline__ void mma_groups(f32x4 (&n)[NG][2], u32x4 (&f)[2][KS],
   }
 }
 
-// Ring protocol.  advance(t) = ring_sync, then the load of chunk t + kN - 1 into the stage chunk t - 1
-// lived in.  A loop calls it once per chunk, in order, before it first touches chunk t; loads are issued
+// Ring protocol.  advance(t) = ring_sync, then the load of the next chunk, t + kN - 1, into the stage
+// chunk t - 1 lived in.  A loop calls it once per chunk, in order, before it first touches chunk t; loads are issued
 // in chunk order, kPer (+1 with an lse row) per wave and chunk, so at that point "all but the newest
 // kN - 2 chunks' loads have arrived" is exactly "chunk t has arrived".  Before the first advance the
 // loads of the first kN - 1 chunks of the sweep have been issued.
@@ -548,9 +572,8 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   Rg rg;
   rg.init(p.k_sr, p.dgran, lane, wave);
   auto stage_of = [&](int t) { return smem + ((uint32_t)t % Rg::kN) * Rg::kStage; };
-  auto issue = [&](int t) {
-    rg.template issue<(STREAM_ONCE ? kLoadOnce : 0)>(kb, p.k_sr, t * kChunk, keys_end, stage_of(t));
-  };
+  rg.start(kb, p.k_sr, c_begin * kChunk, keys_end);
+  auto issue = [&](int t) { rg.template issue_next<(STREAM_ONCE ? kLoadOnce : 0)>(stage_of(t)); };
   auto advance = [&](int t) {
     ring_sync<(Rg::kN - 2) * Rg::kPer>();
     issue(t + Rg::kN - 1);
@@ -609,21 +632,32 @@ __global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
   }
 }
 
-// lse[r] = log2 sum_s 2^part[s][r] over the key ranges of a split row sweep.
+// lse[r] = log2 sum_s 2^part[s][r] over the key ranges of a split row sweep.  One thread per row; the
+// partials are fetched eight at a time (independent loads: a round trip to memory per batch, not per
+// value) and folded into a running (maximum, sum); a NaN partial makes the result NaN.
 __global__ __launch_bounds__(256) void lse_combine_kernel(const float* __restrict__ part, float* __restrict__ lse,
                                                           int64_t rows, int splits) {
   const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
   if (r >= rows) return;
-  float m = kNegInf;
+  float m = kNegInf, acc = 0.f;
   bool nan = false;   // fmaxf drops a NaN partial
-  for (int s = 0; s < splits; ++s) {
-    const float v = part[s * rows + r];
-    nan = nan || (v != v);
-    m = fmaxf(m, v);
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float v[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = (s0 + i < splits) ? part[(int64_t)(s0 + i) * rows + r] : kNegInf;
+    float bm = v[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) bm = fmaxf(bm, v[i]);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) nan = nan || (v[i] != v[i]);
+    const float nm = fmaxf(m, bm);
+    if (nm > kNegInf) {
+      acc *= fast_exp2(m - nm);   // m = -inf: acc is 0 and stays 0
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc += fast_exp2(v[i] - nm);
+      m = nm;
+    }
   }
-  float acc = 0.f;
-  if (m > kNegInf)
-    for (int s = 0; s < splits; ++s) acc += fast_exp2(part[s * rows + r] - m);
   lse[r] = nan ? __builtin_nanf("") : ((m > kNegInf) ? m + fast_log2(acc) : kNegInf);
 }
 
@@ -711,11 +745,16 @@ __global__ __launch_bounds__(kThreads, (NB > 2 ? 1 : 2)) void col_reduce_kernel(
   Rg rg;
   rg.init(p.q_sr, p.dgran, lane, wave);
   auto stage_of = [&](int t) { return smem + ((uint32_t)t % Rg::kN) * Rg::kStage; };
+  rg.start(qb, p.q_sr, t0 * kChunk, p.M);
+  const float* lse_next = lse + t0 * kChunk;   // walks along with the ring's cursor
   auto issue = [&](int t) {
     char* stage = stage_of(t);
-    rg.issue(qb, p.q_sr, t * kChunk, p.M, stage);
-    const __amdgpu_buffer_rsrc_t view = rows_view(reinterpret_cast<const char*>(lse), 4, t * kChunk, p.M);
+    const int live = rows_in_chunk(rg.rows_left);
+    rg.issue_next(stage);
+    const __amdgpu_buffer_rsrc_t view = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(lse_next), 0, live * 4, 0x00020000);
     dma4(view, (uint32_t)lane * 4u, stage + Rg::kRows);   // every wave writes the same 64 values: no branch
+    lse_next += kChunk;
   };
   auto advance = [&](int t) {
     ring_sync<(Rg::kN - 2) * (Rg::kPer + 1)>();
@@ -857,9 +896,10 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
   rg.init(p.k_sr, p.dgran, lane, wave);
   const bool once = p.stream_once != 0;
   auto stage_of = [&](int t) { return smem + ((uint32_t)t % Rg::kN) * Rg::kStage; };
+  rg.start(kb, p.k_sr, c0 * kChunk, keys_end);
   auto issue = [&](int t) {
-    if (once) rg.template issue<kLoadOnce>(kb, p.k_sr, t * kChunk, keys_end, stage_of(t));
-    else rg.template issue<0>(kb, p.k_sr, t * kChunk, keys_end, stage_of(t));
+    if (once) rg.template issue_next<kLoadOnce>(stage_of(t));
+    else rg.template issue_next<0>(stage_of(t));
   };
 #pragma unroll
   for (int i = 0; i < Rg::kN - 1; ++i) issue(c0 + i);

@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define FCR_VERSION 100 /* major*10000 + minor*100 + patch */
+#define FCR_VERSION 200 /* major*10000 + minor*100 + patch */
 
 /* element type of q and k */
 #define FCR_DTYPE_F16 0

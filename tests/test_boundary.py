@@ -34,7 +34,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_version_and_sizes():
     lib = _lib.load()
-    assert lib.fcr_version() == 100
+    assert lib.fcr_version() == 200
     assert lib.fcr_lse_bytes(2, 3, 5, 7, 64) == 2 * 3 * 5 * 4
     assert lib.fcr_lse_bytes(1, 32, 8192, 8192, 128) == 32 * 8192 * 4      # enough row tiles: no scratch
     assert lib.fcr_lse_bytes(1, 32, 128, 4096, 128) == 32 * 128 * 4 * 17   # 16 key ranges + the result
