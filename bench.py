@@ -17,7 +17,8 @@ roofline     the slower of the two kernels, timed alone with events on the launc
 cpu_baseline the CPU oracle (fp32 matmul, mask, softmax, column sum; chunked over query rows)
              timed on this host's cores on a sample of heads of the same workload; the same
              sample is used to check the GPU result against the tolerance of the metric.
-configs      the five named workloads of the benchmark set: ms per call (events), TFLOP/s by the
+configs      the five named workloads of the benchmark set: ms per call (events, after 0.25 s of untimed
+             calls of the same workload), TFLOP/s by the
              metric's convention, fraction of the MFMA (and, for the decode-shaped one, HBM) roofline,
              the CPU oracle timed on a sample of heads, and the tolerance verdict per reduction.
 """
@@ -37,8 +38,9 @@ PEAK_HBM_TBPS = 8.0
 # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # scaled by the same counters on a 256 MiB device copy (FETCH unit 2 KiB, WRITE unit 1 KiB);
 # the summary of those runs is profiles/headline_causal_8192_fp16.md.
-HBM_TRAFFIC_BYTES = {"row_lse_kernel": 198.1e6 + 1.05e6, "col_reduce_kernel": 186.0e6 + 1.05e6}
+HBM_TRAFFIC_BYTES = {"row_lse_kernel": 217.9e6 + 1.05e6, "col_reduce_kernel": 194.9e6 + 1.05e6}
 CONDITIONING_SECONDS = 0.4
+CONFIG_CONDITIONING_SECONDS = 0.25   # per workload and reduction of the configs array, untimed
 
 
 def _events_ms(torch, fn, reps):
@@ -90,8 +92,12 @@ def run_configs(torch, fca, colreduce_ref, inputs, cores):
             got = fn()
             torch.cuda.synchronize()
             reps = 5 if flop > 2e12 else (20 if flop > 1e11 else 100)
-            for _ in range(max(2, reps // 4)):
-                fn()
+            # the CPU oracle ran in between: the same conditioning as for the headline before timing
+            t0 = time.perf_counter()
+            while time.perf_counter() - t0 < CONFIG_CONDITIONING_SECONDS:
+                for _ in range(max(2, reps // 4)):
+                    fn()
+                torch.cuda.synchronize()
             ms = _events_ms(torch, fn, reps)
             cpu_s = None
             for _ in range(1 if flop > 1e11 else 3):
