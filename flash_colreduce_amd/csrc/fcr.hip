@@ -1,24 +1,29 @@
 // libfcr: column reduction of softmax attention for MI355X (gfx950, CDNA4).
 //
-// Two kernels, both built on v_mfma_f32_16x16x32_{f16,bf16} with the product taken as
-// S^T = K * Q^T (keys are MFMA rows, queries are MFMA columns).  In a 16x16 accumulator a lane
-// owns ONE query (lane & 15) and 4 keys (row 4*(lane/16) + r for register r), so
+// Two sweeps, both built on v_mfma_f32_16x16x32_{f16,bf16} (fp32 operands: v_mfma_f32_16x16x4_f32) with
+// the product taken as S^T = K * Q^T (keys are MFMA rows, queries are MFMA columns).  In a 16x16
+// accumulator a lane owns ONE query (lane & 15) and 4 keys (row 4*(lane/16) + r for register r), so
 //   - everything that is per query row (softmax reference exponent, running sum, lse) is one
 //     scalar per lane and needs no cross-lane traffic inside the sweep;
 //   - everything that is per key column accumulates in the lane's registers over the whole
 //     sweep and is reduced across the 16 query lanes once, at the end.
-// The 16x16x32 shape is used because on this chip it sustains about 14 % more flops per watt than
-// 32x32x16 on random operands, and these kernels run against the package power limit.
+// The sweeps are bound by the vector instruction port (an MFMA keeps it for about 10 cycles, the fma,
+// exp2 and add of the 64 scores it produces for 16 more) and, on random operands, by the package power
+// limit.  The 16x16x32 shape is used because the 32x32x16 one, which would halve the MFMAs' share of the
+// port, draws more power on random operands and ends up slower there.
 //
 //   row_lse_kernel    a workgroup keeps 256 query rows in registers (64 per wave; 128 and 32 for
-//                     few or ragged M and for D > 128) and streams key tiles through LDS; writes
-//                     lse2[bh, i] = log2 sum_j 2^(s_ij).
+//                     few or ragged M and for rows longer than 256 bytes) and streams key tiles through
+//                     LDS; writes lse2[bh, i] = log2 sum_j 2^(s_ij).
 //   col_reduce_kernel a workgroup keeps 256 key rows in registers and streams query tiles (and
 //                     their lse2) through LDS; writes out[bh, j] = sum_i or max_i 2^(s_ij-lse2_i).
 //   col_small_kernel  the same result for at most 128 query rows against many keys: queries resident
 //                     in every wave, keys streamed (HBM bound).
-// where s_ij = scale * log2(e) * <q_i, k_j>.  Nothing of size M*N is written anywhere and there
-// are no atomics: one workgroup owns its output rows / columns.
+//   topk_mask_kernel  keep-mask of the k largest columns of every row of the result.
+// where s_ij = scale * log2(e) * <q_i, k_j>.  The streamed operand goes from global memory straight
+// into a swizzled ring of LDS stages (buffer loads with the LDS as destination).  Nothing of size M*N
+// is written anywhere and there are no atomics on global memory: one workgroup owns its output rows /
+// columns.
 //
 // Replaces the Triton kernel of the reference (flash_colreduce/flash.py:11-274).
 
@@ -266,6 +271,14 @@ __device__ __forceinline__ void dma4(__amdgpu_buffer_rsrc_t view, uint32_t byte_
 // all, and no wave is still reading what it read before the barrier, so those stages may be refilled.
 // The empty asm statements keep the compiler from moving LDS accesses across the barrier (there is no
 // fence, which would wait for every outstanding load).
+// A store to LDS that the compiler does not see as one: before a store it does see, it waits for
+// every load-to-LDS in flight (they might write the same bytes), which would drain the ring.  The
+// caller keeps the order: a barrier with lgkmcnt(0) stands between this store and any read of it.
+__device__ __forceinline__ void lds_store_unordered(float* slot, float v) {
+  asm volatile("ds_write_b32 %0, %1" ::"v"((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float*)slot), "v"(v)
+               : "memory");
+}
+
 template <int N>
 __device__ __forceinline__ void ring_sync() {
   asm volatile("" ::: "memory");
@@ -875,7 +888,15 @@ constexpr int kSmallRows = 128;
 template <int DT, int KS, bool CAUSAL, int MODE, int NG>
 __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(const Params p) {
   using Rg = Ring<KS, 3>;   // three workgroups share a CU: 3 x 3 stages of 16 KiB
-  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes];
+  // Finished columns wait in obuf and go to memory kFlush chunks at a time, 1 KiB per store instruction:
+  // up to 10 % faster than a 64-byte store per wave and chunk.  (What the columns cost beyond that does
+  // not depend on how they are stored: 134 MB of them beside 8.6 GB of keys take 15 % of the sweep, which
+  // runs at the row kernel's rate with the stores disabled.)  The ring and obuf are ONE LDS object:
+  // with two, the compiler orders every read of the ring after all loads in flight.
+  constexpr int kFlush = (MODE == kModeBoth) ? 8 : 16;   // 4 KiB of LDS either way
+  constexpr int kObufBytes = (MODE == kModeBoth ? 2 : 1) * kFlush * kChunk * 4;
+  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes + kObufBytes];
+  float* const obuf = reinterpret_cast<float*>(smem + Rg::kBytes);
   int bh, split;
   map_group(p, p.splits, bh, split);
   const int tid = threadIdx.x, lane = tid & 63;
@@ -923,9 +944,29 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
 
   float* out_sum = p.out + (int64_t)bh * p.N;
   float* out_max = ((MODE == kModeBoth) ? p.out2 : p.out) + (int64_t)bh * p.N;
+  float* obuf_max = obuf + (MODE == kModeBoth ? kFlush * kChunk : 0);
+  // Columns of chunks [ta, ta + kFlush) from obuf to memory, up to the end of this workgroup's range;
+  // all waves have passed a barrier since they wrote them.
+  auto flush = [&](int ta) {
+    const int key0 = ta * kChunk, nkeys = keys_end - key0;
+#pragma unroll
+    for (int r = 0; r < kFlush * kChunk / kThreads; ++r) {
+      const int i = tid + r * kThreads;
+      if (i < nkeys) {
+        if (MODE != kModeMax) out_sum[key0 + i] = obuf[i];
+        if (MODE != kModeSum) out_max[key0 + i] = obuf_max[i];
+      }
+    }
+  };
   for (int t = c0; t < c1; ++t) {
     ring_sync<(Rg::kN - 2) * Rg::kPer>();   // chunk t visible, the stage of chunk t - 1 is free
     issue(t + Rg::kN - 1);
+    if (t > c0 && (t - c0) % kFlush == 0) {
+      flush(t - kFlush);
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();   // obuf is free again before anyone writes chunk t's columns
+      asm volatile("" ::: "memory");
+    }
     const char* lds = stage_of(t);
     const int key = t * kChunk + 16 * wave + (lane & 15);
     // query i sees the key iff key <= i + c; chunks that end at or before key c need no mask
@@ -955,18 +996,20 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
         }
     }
     // the four lane groups hold different queries of the same key
+    const int slot = ((t - c0) % kFlush) * kChunk + 16 * wave + lane;
     if (MODE != kModeMax) {
       vsum += __shfl_xor(vsum, 16);
       vsum += __shfl_xor(vsum, 32);
-      if (lane < 16 && key < p.N) out_sum[key] = vsum;
+      if (lane < 16) lds_store_unordered(obuf + slot, vsum);
     }
     if (MODE != kModeSum) {
       vmax = fmaxf(vmax, __shfl_xor(vmax, 16));
       vmax = fmaxf(vmax, __shfl_xor(vmax, 32));
-      if (lane < 16 && key < p.N) out_max[key] = fast_exp2(vmax);
+      if (lane < 16) lds_store_unordered(obuf_max + slot, fast_exp2(vmax));
     }
   }
   ring_sync<0>();   // the loads past the last chunk write their zeros before the LDS is given back
+  flush(c0 + (c1 - c0 - 1) / kFlush * kFlush);
 }
 
 // ---------------------------------------------------------------------------------------------

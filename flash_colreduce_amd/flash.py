@@ -64,8 +64,8 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
 
 def _pack_f32(x: torch.Tensor, is_key: bool) -> torch.Tensor:
     """fp32 operand with D > 128 -> fp16 (see fcr_pack_f32 in include/fcr.h): rows of more than 512
-    bytes do not fit the kernels' resident operand, so these are rounded to fp16 once, which keeps one
-    more mantissa bit than the TF32 rounding the reference's tl.dot applies to fp32 operands
+    bytes do not fit the kernels' resident operand, so these are rounded to fp16 once, which keeps the
+    same 10 explicit mantissa bits as the TF32 rounding the reference's tl.dot applies to fp32 operands
     (flash.py:59,108) but not fp32's range: values beyond +-65504 overflow.  fp32 with D <= 128 never
     comes here: it is multiplied in fp32."""
     b, h, r, d = x.shape
