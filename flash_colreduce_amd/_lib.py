@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libfcr.so")
 
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
-REDUCE_SUM, REDUCE_MAX = 0, 1
+REDUCE_SUM, REDUCE_MAX, REDUCE_MEAN = 0, 1, 2
 
 _I64x4 = ctypes.c_int64 * 4
 _lib = None
@@ -53,6 +53,9 @@ def _declare(lib):
     lib.fcr_colreduce.restype = c.c_int
     lib.fcr_colreduce.argtypes = ([c.c_void_p, c.c_void_p, c.c_void_p, c.c_void_p] + common +
                                   [c.c_int, c.c_int, c.c_void_p])
+    lib.fcr_colreduce_to.restype = c.c_int
+    lib.fcr_colreduce_to.argtypes = ([c.c_void_p, c.c_void_p, c.c_void_p, c.c_int, c.c_void_p] + common +
+                                     [c.c_int, c.c_int, c.c_void_p])
     lib.fcr_colreduce_static.restype = c.c_int
     lib.fcr_colreduce_static.argtypes = ([c.c_void_p, c.c_void_p, c.c_void_p] + common +
                                          [c.c_int, c.c_int, c.c_void_p])

@@ -103,8 +103,8 @@ struct Params {
   float* lse;        // [BH, M]
   float* part;       // [splits, BH, M] partial lse of key ranges when splits > 1
   int splits;        // key ranges per row tile in the row kernel (1 = whole sweep in one workgroup)
-  float* out;        // [BH, N]: column sums (or the only result)
-  float* out2;       // [BH, N]: column maxima when one sweep produces both
+  void* out;         // [BH, N]: column sums or means (or the only result)
+  void* out2;        // [BH, N]: column maxima when one sweep produces both
   int64_t q_sb, q_sh, q_sr;  // strides in BYTES: batch, head, row
   int64_t k_sb, k_sh, k_sr;
   int H, M, N;
@@ -116,6 +116,10 @@ struct Params {
   int group;         // (b,h) pairs whose workgroups are launched together (see map_block)
   int stream_once;   // col_small_kernel: load the keys non-temporally
   int total;         // tiles * B * H workgroups
+  // How the column kernels write a finished column (see store_column)
+  int out_fmt;       // element type of out and out2: FCR_DTYPE_F32, FCR_DTYPE_F16 or FCR_DTYPE_BF16
+  int mean_from;     // < 0: out holds the sums.  Else out holds means: columns below mean_from are
+  float inv_m;       //   multiplied by inv_m = 1/M, column j from there on is divided by N - j
 };
 
 // D[16 keys][16 queries] += A[16 keys][32 d] * B[32 d][16 queries].  Lane l supplies, for A and for
@@ -271,6 +275,39 @@ __device__ __forceinline__ void dma4(__amdgpu_buffer_rsrc_t view, uint32_t byte_
 // all, and no wave is still reading what it read before the barrier, so those stages may be refilled.
 // The empty asm statements keep the compiler from moving LDS accesses across the barrier (there is no
 // fence, which would wait for every outstanding load).
+// The value a float has after a round trip through the result's element type (round to nearest even,
+// overflow to infinity, NaN kept), as the float16_t / bfloat16 casts of torch do it.
+__device__ __forceinline__ float round_trip(int fmt, float v) {
+  if (fmt == FCR_DTYPE_F16) return (float)(_Float16)v;
+  if (fmt == FCR_DTYPE_BF16) {
+    uint32_t b = __builtin_bit_cast(uint32_t, v);
+    b = (v != v) ? 0x7fc00000u : ((b + 0x7fffu + ((b >> 16) & 1u)) & 0xffff0000u);
+    return __builtin_bit_cast(float, b);
+  }
+  return v;
+}
+
+// Writes column `key` of row `bh` of a [BH, N] result whose elements have type p.out_fmt.  The
+// reference casts its fp32 accumulation to the result type first (flash.py:308) and divides the means
+// afterwards, in that type (flash.py:377-384): columns left of the causal offset by the Python scalar
+// M, which torch turns into a multiplication by the fp32 reciprocal, the others by a tensor of counts
+// that torch converts to the result type before the fp32 division.  The same steps, in the same order.
+__device__ __forceinline__ void store_column(const Params& p, void* base, bool is_sum, int bh, int key, float v) {
+  const int fmt = p.out_fmt;
+  if (is_sum && p.mean_from >= 0) {
+    v = round_trip(fmt, v);
+    v = (key < p.mean_from) ? v * p.inv_m : v / round_trip(fmt, (float)(p.N - key));
+  }
+  const int64_t at = (int64_t)bh * p.N + key;
+  if (fmt == FCR_DTYPE_F32) {
+    static_cast<float*>(base)[at] = v;
+  } else if (fmt == FCR_DTYPE_F16) {
+    static_cast<_Float16*>(base)[at] = (_Float16)v;
+  } else {
+    static_cast<uint16_t*>(base)[at] = (uint16_t)(__builtin_bit_cast(uint32_t, round_trip(FCR_DTYPE_BF16, v)) >> 16);
+  }
+}
+
 // A store to LDS that the compiler does not see as one: before a store it does see, it waits for
 // every load-to-LDS in flight (they might write the same bytes), which would drain the ring.  The
 // caller keeps the order: a barrier with lgkmcnt(0) stands between this store and any read of it.
@@ -845,7 +882,7 @@ __global__ __launch_bounds__(kThreads, (NB > 2 ? 1 : 2)) void col_reduce_kernel(
 #pragma unroll
         for (int j = 0; j < 16; ++j) v += src[(j + lane) & 15];
         const int key = k0[grp] + w;
-        if (key < p.N) p.out[(int64_t)bh * p.N + key] = v;
+        if (key < p.N) store_column(p, p.out, true, bh, key, v);
       }
     }
   }
@@ -864,9 +901,8 @@ __global__ __launch_bounds__(kThreads, (NB > 2 ? 1 : 2)) void col_reduce_kernel(
         float v = kNegInf;
 #pragma unroll
         for (int j = 0; j < 16; ++j) v = fmaxf(v, src[(j + lane) & 15]);
-        float* dst = (MODE == kModeBoth) ? p.out2 : p.out;
         const int key = k0[grp] + w;
-        if (key < p.N) dst[(int64_t)bh * p.N + key] = fast_exp2(v);
+        if (key < p.N) store_column(p, (MODE == kModeBoth) ? p.out2 : p.out, false, bh, key, fast_exp2(v));
       }
     }
   }
@@ -942,8 +978,7 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
   u32x4 qf[NG][KS];
   load_resident<KS, NG>(qf, qb, p.q_sr, rows, p.M, p.dgran, lane);
 
-  float* out_sum = p.out + (int64_t)bh * p.N;
-  float* out_max = ((MODE == kModeBoth) ? p.out2 : p.out) + (int64_t)bh * p.N;
+  void* const out_max = (MODE == kModeBoth) ? p.out2 : p.out;
   float* obuf_max = obuf + (MODE == kModeBoth ? kFlush * kChunk : 0);
   // Columns of chunks [ta, ta + kFlush) from obuf to memory, up to the end of this workgroup's range;
   // all waves have passed a barrier since they wrote them.
@@ -953,8 +988,8 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
     for (int r = 0; r < kFlush * kChunk / kThreads; ++r) {
       const int i = tid + r * kThreads;
       if (i < nkeys) {
-        if (MODE != kModeMax) out_sum[key0 + i] = obuf[i];
-        if (MODE != kModeSum) out_max[key0 + i] = obuf_max[i];
+        if (MODE != kModeMax) store_column(p, p.out, true, bh, key0 + i, obuf[i]);
+        if (MODE != kModeSum) store_column(p, out_max, false, bh, key0 + i, obuf_max[i]);
       }
     }
   };
@@ -1362,6 +1397,9 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   p.part = nullptr;
   p.splits = 1;
   p.stream_once = 0;
+  p.out_fmt = FCR_DTYPE_F32;
+  p.mean_from = -1;
+  p.inv_m = 0.f;
   return 0;
 }
 
@@ -1516,9 +1554,15 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
 }
 
 namespace {
-int col_reduce_any(const void* q, const void* k, const float* lse, float* out, float* out2, int mode, int dtype,
+// Element type of the results and whether the sums leave the kernel as means.
+struct ResultSpec {
+  int fmt = FCR_DTYPE_F32;
+  bool mean = false;
+};
+
+int col_reduce_any(const void* q, const void* k, const float* lse, void* out, void* out2, int mode, int dtype,
                    int B, int H, int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
-                   float scale, int causal, void* stream) {
+                   float scale, int causal, void* stream, const ResultSpec& res = ResultSpec()) {
   Params p;
   if (!lse || !out || (mode == kModeBoth && !out2)) return fail(FCR_E_NULL, "null pointer argument");
   int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true, causal != 0, mode);
@@ -1527,6 +1571,11 @@ int col_reduce_any(const void* q, const void* k, const float* lse, float* out, f
   p.lse = const_cast<float*>(lse);
   p.out = out;
   p.out2 = out2;
+  p.out_fmt = res.fmt;
+  if (res.mean) {
+    p.mean_from = causal ? p.c : N;
+    p.inv_m = 1.0f / (float)M;
+  }
   const int ksteps = ksteps_of(dtype, D);
   hipStream_t s = static_cast<hipStream_t>(stream);
   // (fp32 operands always take the general sweep: they are bound by the fp32 matrix rate, not by reading K)
@@ -1647,6 +1696,23 @@ int static_scratch(float** ptr) {
   return 0;
 }
 }  // namespace
+
+int fcr_colreduce_to(const void* q, const void* k, void* out, int out_dtype, float* lse_ws, int dtype, int B, int H,
+                     int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
+                     int reduction, int causal, void* stream) {
+  if (!out || !lse_ws) return fail(FCR_E_NULL, "null pointer argument");
+  if (reduction != FCR_REDUCE_SUM && reduction != FCR_REDUCE_MAX && reduction != FCR_REDUCE_MEAN)
+    return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM, FCR_REDUCE_MAX or FCR_REDUCE_MEAN");
+  if (out_dtype != FCR_DTYPE_F16 && out_dtype != FCR_DTYPE_BF16 && out_dtype != FCR_DTYPE_F32)
+    return fail(FCR_E_DTYPE, "out_dtype must be FCR_DTYPE_F16, FCR_DTYPE_BF16 or FCR_DTYPE_F32");
+  int rc = fcr_row_lse(q, k, lse_ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream);
+  if (rc) return rc;
+  ResultSpec res;
+  res.fmt = out_dtype;
+  res.mean = reduction == FCR_REDUCE_MEAN;
+  return col_reduce_any(q, k, lse_ws, out, nullptr, reduction == FCR_REDUCE_MAX ? kModeMax : kModeSum, dtype, B, H, M,
+                        N, D, q_strides, k_strides, scale, causal, stream, res);
+}
 
 int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, int B, int H, int M, int N, int D,
                          const int64_t q_strides[4], const int64_t k_strides[4], float scale, int reduction,

@@ -80,6 +80,36 @@ def _pack_f32(x: torch.Tensor, is_key: bool) -> torch.Tensor:
     return dst
 
 
+def _operands(query, key):
+    """query and key as the C ABI takes them."""
+    if query.dtype == torch.float32 and (query.shape[3] + 3) // 4 * 16 > _MAX_ROW_BYTES:
+        return _pack_f32(query, False), _pack_f32(key, True)
+    return _device_layout(query), _device_layout(key)
+
+
+_REDUCTIONS = {"sum": _lib.REDUCE_SUM, "max": _lib.REDUCE_MAX, "mean": _lib.REDUCE_MEAN}
+
+
+def _launch_to(query, key, reduction, is_causal, scale, res_dtype):
+    """One reduction, finished on the device: the column kernel stores res_dtype and divides the means
+    (fcr_colreduce_to), so nothing is left for torch to do after the two launches.  Needs M, N, B*H > 0."""
+    b, h, m, d = query.shape
+    n = key.shape[2]
+    if scale is None:
+        scale = 1 / math.sqrt(d)  # the unpadded D (flash.py:366-367)
+    q, k = _operands(query, key)
+    lib = _lib.load()
+    dev = query.device
+    lse = torch.empty(max(b * h * m, lib.fcr_lse_bytes(b, h, m, n, q.shape[3]) // 4), device=dev, dtype=torch.float32)
+    out = torch.empty((b, h, n), device=dev, dtype=res_dtype)
+    with torch.cuda.device(dev):
+        _lib.check(lib.fcr_colreduce_to(q.data_ptr(), k.data_ptr(), out.data_ptr(), _DTYPES[res_dtype], lse.data_ptr(),
+                                        _DTYPES[q.dtype], b, h, m, n, q.shape[3], _lib.strides4(q.stride()),
+                                        _lib.strides4(k.stride()), float(scale), _REDUCTIONS[reduction],
+                                        int(bool(is_causal)), torch.cuda.current_stream(dev).cuda_stream))
+    return out
+
+
 def _launch(query, key, kinds, is_causal, scale):
     """Runs the row kernel once and the column kernel for the entries of `kinds` ('sum' / 'max').
 
@@ -89,11 +119,7 @@ def _launch(query, key, kinds, is_causal, scale):
     n = key.shape[2]
     if scale is None:
         scale = 1 / math.sqrt(d)  # the unpadded D (flash.py:366-367)
-    if query.dtype == torch.float32 and (d + 3) // 4 * 16 > _MAX_ROW_BYTES:
-        q, k = _pack_f32(query, False), _pack_f32(key, True)
-    else:
-        q = _device_layout(query)
-        k = _device_layout(key)
+    q, k = _operands(query, key)
     lib = _lib.load()
     dev = query.device
     # the row statistics, followed by whatever scratch the row kernel wants for this shape
@@ -183,6 +209,8 @@ def flash_colreduce(
     res_dtype = query.dtype if out_dtype is None else out_dtype
     if m == 0 and n > 0 and b * h > 0 and reduction == "max":
         raise ValueError("reduction='max' needs at least one query row.")
+    if m > 0 and b * h * n > 0 and res_dtype in _DTYPES:
+        return _launch_to(query, key, reduction, is_causal, scale, res_dtype)
     if m == 0:
         acc = torch.zeros((b * h, n), device=query.device, dtype=torch.float32)
     else:

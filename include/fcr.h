@@ -42,7 +42,7 @@
 extern "C" {
 #endif
 
-#define FCR_VERSION 200 /* major*10000 + minor*100 + patch */
+#define FCR_VERSION 300 /* major*10000 + minor*100 + patch */
 
 /* element type of q and k */
 #define FCR_DTYPE_F16 0
@@ -52,6 +52,7 @@ extern "C" {
 /* column reduction over query rows */
 #define FCR_REDUCE_SUM 0 /* also the numerator of 'mean' (flash.py:121-122) */
 #define FCR_REDUCE_MAX 1 /* flash.py:123-124 */
+#define FCR_REDUCE_MEAN 2 /* fcr_colreduce_to only: the sums divided as in flash.py:377-384 */
 
 /* argument errors */
 #define FCR_E_NULL -1      /* a required pointer is NULL */
@@ -137,6 +138,20 @@ int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, in
 int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H,
                   int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
                   float scale, int reduction, int causal, void* stream);
+
+/*
+ * The whole operator as the reference's caller sees it: both kernels, the cast of the fp32 accumulation
+ * to the result type (flash.py:308) and, for FCR_REDUCE_MEAN, the division of the sums (flash.py:377-384),
+ * all inside the column kernel's store, so a call is two launches (three when the row sweep splits the
+ * keys) whatever the reduction.  out is [B*H, N] of out_dtype (FCR_DTYPE_F16 / BF16 / F32; the reference
+ * uses the operands' type).  The mean follows the reference's arithmetic step by step: the sum is rounded
+ * to out_dtype first; columns left of the causal offset max(N-M,0) (every column without the mask) are
+ * multiplied by the fp32 reciprocal of M; column j from the offset on is divided by N-j rounded to
+ * out_dtype, the quotient rounded to out_dtype.  lse_ws as for fcr_colreduce.
+ */
+int fcr_colreduce_to(const void* q, const void* k, void* out, int out_dtype, float* lse_ws, int dtype, int B,
+                     int H, int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
+                     float scale, int reduction, int causal, void* stream);
 
 /*
  * fcr_colreduce without the lse_ws argument, for callers that cannot allocate device memory (code under

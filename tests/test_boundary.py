@@ -27,14 +27,14 @@ def test_library_exports_every_declared_symbol():
     names = _declared_symbols()
     assert {"fcr_version", "fcr_last_error", "fcr_lse_bytes", "fcr_row_lse", "fcr_col_reduce",
             "fcr_col_reduce_sum_max", "fcr_pack_f32", "fcr_colreduce", "fcr_colreduce_static",
-            "fcr_topk_mask"} <= set(names)
+            "fcr_colreduce_to", "fcr_topk_mask"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
 
 
 def test_version_and_sizes():
     lib = _lib.load()
-    assert lib.fcr_version() == 200
+    assert lib.fcr_version() == 300
     assert lib.fcr_lse_bytes(2, 3, 5, 7, 64) == 2 * 3 * 5 * 4
     assert lib.fcr_lse_bytes(1, 32, 8192, 8192, 128) == 32 * 8192 * 4      # enough row tiles: no scratch
     assert lib.fcr_lse_bytes(1, 32, 128, 4096, 128) == 32 * 128 * 4 * 17   # 16 key ranges + the result
@@ -52,10 +52,13 @@ def _call(lib, fn, **over):
         return lib.fcr_row_lse(a["q"], a["k"], a["lse"], *common, a["causal"], None)
     if fn == "col_reduce":
         return lib.fcr_col_reduce(a["q"], a["k"], a["lse"], a["out"], *common, a["red"], a["causal"], None)
+    if fn == "colreduce_to":
+        return lib.fcr_colreduce_to(a["q"], a["k"], a["out"], a.get("out_dtype", 0), a["lse"], *common, a["red"],
+                                    a["causal"], None)
     return lib.fcr_colreduce(a["q"], a["k"], a["out"], a["lse"], *common, a["red"], a["causal"], None)
 
 
-@pytest.mark.parametrize("fn", ["row_lse", "col_reduce", "colreduce"])
+@pytest.mark.parametrize("fn", ["row_lse", "col_reduce", "colreduce", "colreduce_to"])
 def test_c_abi_rejects_bad_arguments_without_a_device(fn):
     """Every rejection happens before the first HIP call, so fake pointers are safe here."""
     lib = _lib.load()
@@ -71,7 +74,10 @@ def test_c_abi_rejects_bad_arguments_without_a_device(fn):
         (dict(qs=(512, 512, 0, 1)), -4), (dict(ks=(512, 512, 32, 1)), -4),   # overlapping rows
         (dict(scale=float("inf")), -6), (dict(scale=float("nan")), -6),
     ]
-    if fn != "row_lse":
+    if fn == "colreduce_to":   # takes the mean as a third reduction, and a result type
+        cases += [(dict(out=None), -1), (dict(red=3), -5), (dict(red=-1), -5), (dict(out_dtype=3), -2),
+                  (dict(out_dtype=-1), -2)]
+    elif fn != "row_lse":
         cases += [(dict(out=None), -1), (dict(red=2), -5), (dict(red=-1), -5)]
     for over, code in cases:
         assert _call(lib, fn, **over) == code, over

@@ -464,6 +464,34 @@ def test_output_dtype_and_mean_epilogue():
     torch.testing.assert_close(out, (s / div.to(torch.bfloat16)), rtol=0, atol=0)
 
 
+@pytest.mark.parametrize("res_dtype", [None, torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n,d,dtype", [(300, 5000, 64, torch.bfloat16),     # counts that bf16 and fp16 round
+                                         (700, 300, 128, torch.float16),     # more queries than keys
+                                         (40, 9000, 128, torch.float16),     # the few-queries column sweep
+                                         (1, 77, 32, torch.bfloat16), (513, 513, 72, torch.float16)])
+def test_cast_and_mean_in_the_kernel_repeat_the_torch_steps(m, n, d, dtype, causal, res_dtype):
+    """The column kernel's typed store against the reference's own sequence of torch operations
+    (flash.py:308 cast, 377-384 in-place divisions) applied to the fp32 result of the C ABI: bit for bit."""
+    from flash_colreduce_amd import flash as F
+    q, k = _inputs.randn_pair(2, 3, m, n, d, seed=m + n, dtype=dtype)
+    q, k = q.cuda(), k.cuda()
+    want_dtype = dtype if res_dtype is None else res_dtype
+    for red in REDUCTIONS:
+        got = fca.flash_colreduce(q, k, red, is_causal=causal, out_dtype=res_dtype)
+        (acc,), _ = F._launch(q, k, ["max" if red == "max" else "sum"], causal, None)
+        scores = acc.view(2, 3, n).to(want_dtype)
+        if red == "mean":
+            if causal:
+                c = max(n - m, 0)
+                scores[..., :c] /= m
+                scores[..., c:] /= torch.arange(n - c, 0, -1, device=q.device)
+            else:
+                scores /= m
+        assert got.dtype == want_dtype and got.shape == (2, 3, n)
+        assert torch.equal(got, scores), (red, (got.float() - scores.float()).abs().max().item())
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_multi_reduction_shares_the_row_pass(causal):
     q, k = _inputs.randn_pair(2, 3, 300, 450, 64, seed=8, dtype=torch.bfloat16)
