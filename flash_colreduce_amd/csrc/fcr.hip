@@ -1311,6 +1311,194 @@ __global__ __launch_bounds__(kTopkThreads) void topk_mask_long_kernel(const floa
 }
 
 // ---------------------------------------------------------------------------------------------
+// Rows of more than 32768 columns with a workspace: a row is spread over workgroups of VPT * 1024
+// columns (VPT = 32 keys per thread, in registers, when that still gives a workgroup per CU, else 8).  Radix select, eight bits per launch: launch PASS
+// histograms digit PASS of the keys that match the digits chosen so far, one histogram per workgroup,
+// written whole (no atomics in memory, nothing to clear, bitwise reproducible).  Every workgroup of the
+// next launch adds up the row's histograms and repeats the choice of the digit, so no launch is needed
+// for that.  The last launch chooses the fourth digit, finds the ties in front of its columns in the
+// earlier workgroups' histograms of that digit, and writes the mask.
+
+struct TopkState {
+  uint32_t prefix;   // digits chosen so far, in place
+  uint32_t need;     // how many keys to keep among those that match the prefix
+  uint32_t ties;     // how many keys fell into the digit chosen last
+  uint32_t pad;
+};
+
+// workspace: hist[2][rows][parts][256] followed by state[rows][4]
+__host__ __device__ inline size_t topk_hist_words(int64_t rows, int parts) { return (size_t)rows * parts * 256; }
+
+// The choice of digit `pass` for one row, by the whole workgroup: the bins of the row's `parts` histograms
+// are added up, then one wave walks them from the top.  prev is the state before this digit.
+__device__ __forceinline__ TopkState topk_choose(const uint32_t* __restrict__ hist_row, int parts, TopkState prev,
+                                                 int pass, uint32_t* bins, TopkState* chosen, int tid, int lane) {
+  const int shift = 24 - 8 * pass;
+  if (tid < 256) {
+    uint32_t v = 0;
+    for (int q = 0; q < parts; ++q) v += hist_row[q * 256 + tid];
+    bins[tid] = v;
+  }
+  if (tid == 0) *chosen = TopkState{prev.prefix | (0xffu << shift), 0u, 0u, 0u};   // need == 0: nothing is kept
+  __syncthreads();
+  if (tid < 64) {   // 4 bins per lane, lane 0 holds the four largest digits; suffix sums across lanes
+    uint32_t h[4], tot = 0;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      h[e] = bins[255 - (lane * 4 + e)];
+      tot += h[e];
+    }
+    uint32_t incl = tot;
+#pragma unroll
+    for (int dd = 1; dd < 64; dd <<= 1) {
+      const uint32_t o = __shfl_up(incl, dd);
+      if (lane >= dd) incl += o;
+    }
+    uint32_t above = incl - tot;   // keys in larger digits than this lane's
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (above < prev.need && above + h[e] >= prev.need)   // true for exactly one bin when need > 0
+        *chosen = TopkState{prev.prefix | ((uint32_t)(255 - (lane * 4 + e)) << shift), prev.need - above, h[e], 0u};
+      above += h[e];
+    }
+  }
+  __syncthreads();
+  const TopkState out = *chosen;
+  __syncthreads();   // bins and chosen may be written again
+  return out;
+}
+
+// The VPT keys of a thread from column col0 on; columns past N get key 0 and valid bit 0.
+template <int VPT>
+__device__ __forceinline__ uint32_t topk_load(const float* __restrict__ s, int N, int col0, bool vec, uint32_t u[VPT]) {
+  if (vec && col0 + VPT <= N) {
+#pragma unroll
+    for (int i = 0; i < VPT; i += 4) {
+      const f32x4 a = *reinterpret_cast<const f32x4*>(s + col0 + i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) u[i + e] = order_key(a[e]);
+    }
+    return VPT == 32 ? 0xffffffffu : (1u << (VPT & 31)) - 1u;
+  }
+  uint32_t valid = 0;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const bool in = col0 + i < N;
+    u[i] = in ? order_key(s[in ? col0 + i : 0]) : 0u;
+    valid |= in ? (1u << i) : 0u;
+  }
+  return valid;
+}
+
+template <int PASS, int VPT>
+__global__ __launch_bounds__(kTopkThreads) void topk_spread_hist_kernel(const float* __restrict__ scores,
+                                                                        uint32_t* __restrict__ ws, int64_t rows,
+                                                                        int N, int k, int parts) {
+  __shared__ uint32_t bins[256];
+  __shared__ uint32_t hist[256];
+  __shared__ TopkState chosen;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int64_t row = blockIdx.x / parts;
+  const int part = (int)(blockIdx.x - row * parts);
+  const size_t words = topk_hist_words(rows, parts);
+  TopkState* states = reinterpret_cast<TopkState*>(ws + 2 * words) + row * 4;
+  uint32_t* mine = ws + (PASS & 1) * words + ((size_t)row * parts + part) * 256;
+
+  uint32_t u[VPT];
+  const float* s = scores + row * N;
+  const bool vec = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0;
+  const uint32_t valid = topk_load<VPT>(s, N, (part * kTopkThreads + tid) * VPT, vec, u);
+
+  TopkState st{0u, (uint32_t)min(max(k, 0), N), 0u, 0u};
+  if (PASS > 0) {
+    if (PASS > 1) st = states[PASS - 2];
+    st = topk_choose(ws + ((PASS - 1) & 1) * words + (size_t)row * parts * 256, parts, st, PASS - 1, bins, &chosen,
+                     tid, lane);
+    if (part == 0 && tid == 0) states[PASS - 1] = st;
+  }
+  if (tid < 256) hist[tid] = 0;
+  __syncthreads();
+  constexpr uint32_t decided = PASS == 0 ? 0u : 0xffffffffu << (32 - 8 * PASS);
+  constexpr int shift = 24 - 8 * PASS;
+#pragma unroll
+  for (int i = 0; i < VPT; ++i) {
+    const bool live = ((valid >> i) & 1u) && ((u[i] & decided) == st.prefix);
+    const uint32_t d = (u[i] >> shift) & 255u;
+    const uint64_t lives = __builtin_amdgcn_ballot_w64(live);
+    if (lives == 0) continue;
+    const uint32_t d0 = __builtin_amdgcn_readlane(d, __builtin_ctzll(lives));
+    if (__builtin_amdgcn_ballot_w64(live && d == d0) == lives) {   // one bin for the whole wave
+      if (lane == 0) atomicAdd(&hist[d0], (uint32_t)__builtin_popcountll(lives));
+    } else if (live) {
+      atomicAdd(&hist[d], 1u);
+    }
+  }
+  __syncthreads();
+  if (tid < 256) mine[tid] = hist[tid];
+}
+
+template <int VPT>
+__global__ __launch_bounds__(kTopkThreads) void topk_spread_write_kernel(const float* __restrict__ scores,
+                                                                         uint8_t* __restrict__ mask,
+                                                                         float* __restrict__ threshold,
+                                                                         const uint32_t* __restrict__ ws, int64_t rows,
+                                                                         int N, int k, int parts) {
+  constexpr int kW = kTopkThreads / 64;
+  __shared__ uint32_t bins[256];
+  __shared__ TopkState chosen;
+  __shared__ uint32_t wave_eq[kW];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int64_t row = blockIdx.x / parts;
+  const int part = (int)(blockIdx.x - row * parts);
+  const size_t words = topk_hist_words(rows, parts);
+  const TopkState* states = reinterpret_cast<const TopkState*>(ws + 2 * words) + row * 4;
+  const uint32_t* last = ws + words + (size_t)row * parts * 256;   // the histograms of digit 3 (3 & 1 == 1)
+
+  uint32_t u[VPT];
+  const float* s = scores + row * N;
+  const bool vec = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0;
+  const int col0 = (part * kTopkThreads + tid) * VPT;
+  const uint32_t valid = topk_load<VPT>(s, N, col0, vec, u);
+
+  const uint32_t kk = (uint32_t)min(max(k, 0), N);
+  const TopkState st = topk_choose(last, parts, states[2], 3, bins, &chosen, tid, lane);
+  const uint32_t T = st.prefix, need = st.need, ties = (kk > 0) ? st.ties : 0u;
+  if (part == 0 && tid == 0 && threshold) threshold[row] = key_value(T);
+
+  uint32_t before = 0;
+  if (need < ties) {   // uniform over the row: some ties are dropped, rank them by column
+    uint32_t mine = 0;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) mine += (((valid >> i) & 1u) && u[i] == T) ? 1u : 0u;
+    before = ties_before(mine, wave_eq, lane, wave);
+    for (int q = 0; q < part; ++q) before += last[q * 256 + (T & 255u)];   // ties in the workgroups in front
+  }
+  const bool keep_all_ties = need >= ties;
+  uint8_t* m = mask + row * N;
+  const bool whole = valid == (VPT == 32 ? 0xffffffffu : (1u << (VPT & 31)) - 1u) && (N & 7) == 0 &&
+                     (reinterpret_cast<uintptr_t>(mask) & 7) == 0;
+#pragma unroll
+  for (int i0 = 0; i0 < VPT; i0 += 8) {
+    uint64_t w = 0;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const int i = i0 + e;
+      const bool eq = ((valid >> i) & 1u) && u[i] == T;
+      const bool keep = (kk > 0) && ((u[i] > T) || (eq && (keep_all_ties || before < need)));
+      if (eq) ++before;
+      w |= (uint64_t)(keep ? 1 : 0) << (8 * e);
+    }
+    if (whole) {
+      *reinterpret_cast<uint64_t*>(m + col0 + i0) = w;
+    } else {
+#pragma unroll
+      for (int e = 0; e < 8; ++e)
+        if ((valid >> (i0 + e)) & 1u) m[col0 + i0 + e] = (uint8_t)(w >> (8 * e));
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------------------------
 thread_local char g_err[256] = "";
 
 int fail(int code, const char* what) {
@@ -1507,6 +1695,20 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
 
 }  // namespace
 
+namespace {
+template <int VPT>
+void launch_topk_spread(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, uint32_t* w,
+                        hipStream_t s) {
+  const int parts = (N + VPT * kTopkThreads - 1) / (VPT * kTopkThreads);
+  const dim3 grid((unsigned)(rows * parts)), block(kTopkThreads);
+  hipLaunchKernelGGL((topk_spread_hist_kernel<0, VPT>), grid, block, 0, s, scores, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_hist_kernel<1, VPT>), grid, block, 0, s, scores, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_hist_kernel<2, VPT>), grid, block, 0, s, scores, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_hist_kernel<3, VPT>), grid, block, 0, s, scores, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_write_kernel<VPT>), grid, block, 0, s, scores, mask, threshold, w, rows, N, k, parts);
+}
+}  // namespace
+
 extern "C" {
 
 int fcr_version(void) { return FCR_VERSION; }
@@ -1628,6 +1830,28 @@ int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float
                            const int64_t k_strides[4], float scale, int causal, void* stream) {
   return col_reduce_any(q, k, lse, out_sum, out_max, kModeBoth, dtype, B, H, M, N, D, q_strides, k_strides, scale,
                         causal, stream);
+}
+
+size_t fcr_topk_bytes(int64_t rows, int N) {
+  if (rows < 1 || N <= 32 * kTopkThreads || N > (1 << 30)) return 0;
+  const int parts = (N + 8 * kTopkThreads - 1) / (8 * kTopkThreads);   // the finer of the two ways to cut a row
+  if (rows * parts > 0x7fffffffll) return 0;
+  return 2 * topk_hist_words(rows, parts) * sizeof(uint32_t) + (size_t)rows * 4 * sizeof(TopkState);
+}
+
+int fcr_topk_mask_ws(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* ws,
+                     size_t ws_bytes, void* stream) {
+  const size_t want = fcr_topk_bytes(rows, N);
+  if (!ws || want == 0 || ws_bytes < want) return fcr_topk_mask(scores, mask, threshold, rows, N, k, stream);
+  if (!scores || !mask) return fail(FCR_E_NULL, "null pointer argument");
+  if ((reinterpret_cast<uintptr_t>(ws) & 15) != 0) return fail(FCR_E_STRIDE, "the top-k workspace must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  uint32_t* w = static_cast<uint32_t*>(ws);
+  // 32 keys per thread while that leaves a workgroup per CU, else 8
+  const int64_t coarse = rows * ((N + 32 * kTopkThreads - 1) / (32 * kTopkThreads));
+  if (coarse >= chip_cus()) launch_topk_spread<32>(scores, mask, threshold, rows, N, k, w, s);
+  else launch_topk_spread<8>(scores, mask, threshold, rows, N, k, w, s);
+  return launched("topk_spread kernels");
 }
 
 int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream) {

@@ -293,7 +293,11 @@ def topk_keep_mask(scores: torch.Tensor, k: int, return_threshold: bool = False)
         mask = torch.zeros(s.shape, device=s.device, dtype=torch.bool)
     thr = torch.empty(s.shape[:-1], device=s.device, dtype=torch.float32) if return_threshold else None
     if rows > 0 and n > 0:
+        lib = _lib.load()
+        nbytes = lib.fcr_topk_bytes(rows, n)   # > 0 for long rows: scratch that lets workgroups share a row
+        ws = torch.empty(nbytes, device=s.device, dtype=torch.uint8) if nbytes else None
         with torch.cuda.device(s.device):
-            _lib.check(_lib.load().fcr_topk_mask(s.data_ptr(), mask.data_ptr(), thr.data_ptr() if thr is not None else None,
-                                                 rows, n, int(k), torch.cuda.current_stream(s.device).cuda_stream))
+            _lib.check(lib.fcr_topk_mask_ws(s.data_ptr(), mask.data_ptr(), thr.data_ptr() if thr is not None else None,
+                                            rows, n, int(k), ws.data_ptr() if ws is not None else None, nbytes,
+                                            torch.cuda.current_stream(s.device).cuda_stream))
     return (mask, thr) if return_threshold else mask

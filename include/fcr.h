@@ -119,6 +119,17 @@ int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float
 int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream);
 
 /*
+ * fcr_topk_mask with scratch memory, for long rows: with ws_bytes >= fcr_topk_bytes(rows, N) > 0 a row of
+ * more than 32768 columns is spread over workgroups of 8192 columns (five launches: four digits of a
+ * radix select, then the mask) instead of being walked by one workgroup; same result, bit for bit.
+ * fcr_topk_bytes returns 0 where the scratch would not be used (N <= 32768); with ws NULL or too small
+ * the call is fcr_topk_mask.  ws must be 16-byte aligned; its contents before and after are irrelevant.
+ */
+size_t fcr_topk_bytes(int64_t rows, int N);
+int fcr_topk_mask_ws(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* ws,
+                     size_t ws_bytes, void* stream);
+
+/*
  * fp32 operands with D > 128, or as a faster and less exact alternative to FCR_DTYPE_F32 (values must
  * fit fp16): packs a contiguous fp32 [rows, D] into the fp16 [rows, terms * Dp] (Dp = D rounded up
  * to 8, zero padded) that the kernels above take with D' = terms * Dp and dtype FCR_DTYPE_F16.

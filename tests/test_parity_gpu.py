@@ -548,6 +548,39 @@ def test_topk_keep_mask(n, k):
         assert torch.equal(thr.view(6).cpu(), kth)
 
 
+@pytest.mark.parametrize("rows,n,k", [(5, 32769, 5), (5, 40000, 39999), (5, 70001, 1234), (5, 262144, 65536),
+                                      (5, 300007, 100000),
+                                      (128, 65537, 3000), (64, 131072, 131000)])   # 32 keys per thread
+def test_topk_long_rows_with_and_without_scratch(rows, n, k):
+    """Rows of more than 32768 columns: spread over workgroups when the caller brings scratch
+    (fcr_topk_mask_ws), one workgroup per row otherwise (fcr_topk_mask); both against the oracle."""
+    from flash_colreduce_amd import _lib
+    from oracle.colreduce_oracle import topk_mask_ref
+    g = torch.Generator().manual_seed(n)
+    vals = torch.randn(rows, n, generator=g)
+    vals[1] = (vals[1] * 4).round() / 4           # heavy ties, both signs
+    vals[2] = 1.5                                 # all equal: the lowest k columns win
+    vals[3, : n // 2] = vals[3, n // 2: n // 2 * 2]   # every value of the first half twice
+    want = topk_mask_ref(vals.numpy(), k)
+    kth = torch.sort(vals, dim=1, descending=True).values[:, k - 1]
+    lib = _lib.load()
+    dev = vals.cuda()
+    stream = torch.cuda.current_stream().cuda_stream
+    nbytes = lib.fcr_topk_bytes(rows, n)
+    assert nbytes > 0 and lib.fcr_topk_bytes(rows, 32768) == 0
+    ws = torch.full((nbytes,), 0xAB, device="cuda", dtype=torch.uint8)   # the scratch need not be cleared
+    for use_ws in (True, False):
+        mask = torch.full((rows, n), 7, device="cuda", dtype=torch.uint8)
+        thr = torch.empty(rows, device="cuda")
+        if use_ws:
+            _lib.check(lib.fcr_topk_mask_ws(dev.data_ptr(), mask.data_ptr(), thr.data_ptr(), rows, n, k, ws.data_ptr(),
+                                            nbytes, stream))
+        else:
+            _lib.check(lib.fcr_topk_mask(dev.data_ptr(), mask.data_ptr(), thr.data_ptr(), rows, n, k, stream))
+        assert (mask.cpu().numpy() == want).all(), use_ws
+        assert torch.equal(thr.cpu(), kth), use_ws
+
+
 def test_topk_on_reduced_columns():
     from oracle.colreduce_oracle import topk_mask_ref
     q, k = _inputs.config4(heads=4, n=2048)
