@@ -95,7 +95,7 @@ def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None)
 
 
 TOPK_SHAPES = ((32, 8192, 2048), (32, 8192, 64), (32, 32768, 8192), (32, 32768, 512), (256, 8192, 2048),
-               (32, 262144, 65536))
+               (32, 262144, 65536), (8, 1048576, 100000))
 
 
 def run_topk(out=sys.stdout):

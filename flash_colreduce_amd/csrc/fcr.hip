@@ -19,8 +19,10 @@
 //                     their lse2) through LDS; writes out[bh, j] = sum_i or max_i 2^(s_ij-lse2_i).
 //   col_small_kernel  the same result for at most 128 query rows against many keys: queries resident
 //                     in every wave, keys streamed (HBM bound).
-//   topk_mask_kernel  keep-mask of the k largest columns of every row of the result.
-// where s_ij = scale * log2(e) * <q_i, k_j>.  The streamed operand goes from global memory straight
+//   topk_mask_kernel  keep-mask of the k largest columns of every row of the result (one workgroup per
+//                     row; topk_spread_* kernels share a long row between workgroups).
+// where s_ij = scale * log2(e) * <q_i, k_j>.  The column kernels store the result type of the caller's choice
+// and divide the means as they store (store_column).  The streamed operand goes from global memory straight
 // into a swizzled ring of LDS stages (buffer loads with the LDS as destination).  Nothing of size M*N
 // is written anywhere and there are no atomics on global memory: one workgroup owns its output rows /
 // columns.
