@@ -751,8 +751,10 @@ inline int col_tile_blocks(int ksteps, int mode, int N, int64_t bh, bool causal)
   if (nb != 2) return nb;
   const int64_t wgs2 = bh * ((N + kWaves * 64 - 1) / (kWaves * 64));
   const int cus = chip_cus();
-  if (causal) return (wgs2 >= cus && wgs2 <= 2 * cus) ? 1 : 2;
-  return (wgs2 > cus && wgs2 < 2 * cus) ? 1 : 2;
+  // two-block tiles only when they still give two workgroups per CU; with fewer, CUs idle or run a single
+  // workgroup (32 heads of 1024 x 1024: the call takes 37 us with 128 two-block tiles, 32 us with 256 one-block tiles)
+  if (causal) return wgs2 <= 2 * cus ? 1 : 2;
+  return wgs2 < 2 * cus ? 1 : 2;
 }
 
 template <int DT, int KS, bool CAUSAL, int MODE, int NB>
