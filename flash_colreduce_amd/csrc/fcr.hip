@@ -94,7 +94,8 @@ inline int row_blocks_per_wave(int ksteps, int M, int64_t bh, bool causal) {
 inline int row_tile_rows(int ksteps, int M, int64_t bh, bool causal) {
   return kWaves * 32 * row_blocks_per_wave(ksteps, M, bh, causal);
 }
-constexpr int kMaxKSteps = 8;                 // D <= 256
+constexpr int kMaxKSteps = 8;                 // 16-bit elements: D <= 256
+constexpr int kMaxKStepsF32 = 16;             // fp32: D <= 256 as well (rows of up to 1 KiB, one workgroup per CU)
 constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row sub-steps)
 constexpr float kNegInf = -__builtin_inff();
 constexpr float kPosInf = __builtin_inff();
@@ -338,7 +339,7 @@ __device__ __forceinline__ int rows_in_chunk(int rows_left) {
 template <int KS, int NS = ring_stages(KS)>
 struct Ring {
   static constexpr int kN = NS;
-  static constexpr int kPitch = KS <= 1 ? 64 : KS == 2 ? 128 : KS <= 4 ? 256 : 512;   // LDS row pitch
+  static constexpr int kPitch = KS <= 1 ? 64 : KS == 2 ? 128 : KS <= 4 ? 256 : KS <= 8 ? 512 : 1024;   // LDS row pitch
   static constexpr int kRowsPerLoad = 1024 / kPitch;                 // rows one wave-wide load covers
   static constexpr int kPer = kChunk / (kWaves * kRowsPerLoad);     // loads per wave and chunk
   static constexpr int kRows = kChunk * kPitch;                      // bytes of rows in a stage
@@ -583,7 +584,7 @@ struct NoAux {};
 // non-temporally (7.0 instead of 6.2 TB/s on 34 GB of keys).  With several row tiles, or few keys, the
 // default policy is the faster one.
 template <int DT, int KS, bool CAUSAL, int NB, bool STREAM_ONCE>
-__global__ __launch_bounds__(kThreads, 2) void row_lse_kernel(const Params p) {
+__global__ __launch_bounds__(kThreads, (KS > 8 ? 1 : 2)) void row_lse_kernel(const Params p) {
   using Rg = Ring<KS>;
   constexpr int NG = 2 * NB;
   constexpr int kTileRows = kWaves * 32 * NB;
@@ -758,7 +759,7 @@ inline int col_tile_blocks(int ksteps, int mode, int N, int64_t bh, bool causal)
 }
 
 template <int DT, int KS, bool CAUSAL, int MODE, int NB>
-__global__ __launch_bounds__(kThreads, (NB > 2 ? 1 : 2)) void col_reduce_kernel(const Params p) {
+__global__ __launch_bounds__(kThreads, ((NB > 2 || KS > 8) ? 1 : 2)) void col_reduce_kernel(const Params p) {
   using Rg = Ring<KS>;
   constexpr int NG = 2 * NB;
   constexpr int kTileRows = kWaves * 32 * NB;
@@ -1557,9 +1558,9 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
     return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16, FCR_DTYPE_BF16 or FCR_DTYPE_F32");
   if (B < 1 || H < 1 || M < 1 || N < 1) return fail(FCR_E_SHAPE, "B, H, M, N must be >= 1");
   const int esize = elem_bytes(dtype);
-  if (D < 1 || D > 64 * kMaxKSteps / esize || (D * esize) % 16 != 0)
+  if (D < 1 || D > 256 || (D * esize) % 16 != 0)
     return fail(FCR_E_SHAPE, esize == 2 ? "D must be a multiple of 8 in [8, 256]"
-                                         : "D must be a multiple of 4 in [4, 128] for FCR_DTYPE_F32");
+                                         : "D must be a multiple of 4 in [4, 256] for FCR_DTYPE_F32");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
   if (bh * (((int64_t)(by_keys ? N : M) + 127) / 128) > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
@@ -1689,6 +1690,20 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
     default: CALL(DT, 8); break;                           \
   }
 
+// fp32 rows are twice as long: up to 16 k-steps
+#define FCR_DISPATCH_KS_F32(ksteps, CALL)                         \
+  switch (ksteps) {                                               \
+    case 9: CALL(FCR_DTYPE_F32, 9); break;                        \
+    case 10: CALL(FCR_DTYPE_F32, 10); break;                      \
+    case 11: CALL(FCR_DTYPE_F32, 11); break;                      \
+    case 12: CALL(FCR_DTYPE_F32, 12); break;                      \
+    case 13: CALL(FCR_DTYPE_F32, 13); break;                      \
+    case 14: CALL(FCR_DTYPE_F32, 14); break;                      \
+    case 15: CALL(FCR_DTYPE_F32, 15); break;                      \
+    case 16: CALL(FCR_DTYPE_F32, 16); break;                      \
+    default: FCR_DISPATCH_KS(FCR_DTYPE_F32, ksteps, CALL)         \
+  }
+
 #define FCR_DISPATCH_KS4(DT, ksteps, CALL)                 \
   switch (ksteps) {                                        \
     case 1: CALL(DT, 1); break;                            \
@@ -1724,7 +1739,7 @@ size_t fcr_lse_bytes(int B, int H, int M, int N, int D) {
   // the most any row width asks for (the tile height, hence the split count, depends a little on the
   // number of 64-byte k-steps of a row), so the size holds for every dtype and D
   int splits = 1;
-  for (int ks = 1; ks <= kMaxKSteps; ++ks) {
+  for (int ks = 1; ks <= kMaxKStepsF32; ++ks) {
     const int s = row_splits(B, H, M, N, ks);
     if (s > splits) splits = s;
   }
@@ -1749,7 +1764,7 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
 #define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal != 0, s)
   if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_LSE) }
   else if (dtype == FCR_DTYPE_BF16) { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_LSE) }
-  else { FCR_DISPATCH_KS(FCR_DTYPE_F32, ksteps, FCR_CALL_LSE) }
+  else { FCR_DISPATCH_KS_F32(ksteps, FCR_CALL_LSE) }
 #undef FCR_CALL_LSE
   rc = launched("row_lse_kernel");
   if (rc || p.splits == 1) return rc;
@@ -1814,7 +1829,7 @@ int col_reduce_any(const void* q, const void* k, const float* lse, void* out, vo
 #define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal != 0, mode, s)
   if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_COL) }
   else if (dtype == FCR_DTYPE_BF16) { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL) }
-  else { FCR_DISPATCH_KS(FCR_DTYPE_F32, ksteps, FCR_CALL_COL) }
+  else { FCR_DISPATCH_KS_F32(ksteps, FCR_CALL_COL) }
 #undef FCR_CALL_COL
   return launched("col_reduce_kernel");
 }

@@ -16,7 +16,6 @@ from . import _lib
 __all__ = ["flash_colreduce", "flash_colreduce_multi", "row_lse2", "topk_keep_mask"]
 
 _DTYPES = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_F32}
-_MAX_ROW_BYTES = 512   # a row the kernels can hold: D <= 256 for 16-bit elements, <= 128 for fp32
 
 
 def _validate(query: torch.Tensor, key: torch.Tensor, reduction: Optional[str]):
@@ -62,15 +61,13 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
     return x.clone(memory_format=torch.contiguous_format) if x.is_contiguous() else x.contiguous()
 
 
-def _pack_f32(x: torch.Tensor, is_key: bool) -> torch.Tensor:
-    """fp32 operand with D > 128 -> fp16 (see fcr_pack_f32 in include/fcr.h): rows of more than 512
-    bytes do not fit the kernels' resident operand, so these are rounded to fp16 once, which keeps the
-    same 10 explicit mantissa bits as the TF32 rounding the reference's tl.dot applies to fp32 operands
-    (flash.py:59,108) but not fp32's range: values beyond +-65504 overflow.  fp32 with D <= 128 never
-    comes here: it is multiplied in fp32."""
+def pack_f32(x: torch.Tensor, is_key: bool, terms: int = 3) -> torch.Tensor:
+    """fp32 (B,H,R,D) -> the fp16 segments of fcr_pack_f32 (include/fcr.h), for callers of the C ABI that
+    want fp32 operands multiplied on the 16-bit matrix instructions (16 times the fp32 rate) and accept
+    fp16's range: terms = 3 gives products to about 2^-22 and needs 3 * ceil8(D) <= 256, terms = 1 is one
+    rounding to fp16.  flash_colreduce itself never comes here: it multiplies fp32 operands in fp32."""
     b, h, r, d = x.shape
     dpad = (d + 7) // 8 * 8
-    terms = 3 if 3 * dpad <= 256 else 1
     src = x.contiguous()
     dst = torch.empty((b, h, r, terms * dpad), device=x.device, dtype=torch.float16)
     if dst.numel():
@@ -82,8 +79,6 @@ def _pack_f32(x: torch.Tensor, is_key: bool) -> torch.Tensor:
 
 def _operands(query, key):
     """query and key as the C ABI takes them."""
-    if query.dtype == torch.float32 and (query.shape[3] + 3) // 4 * 16 > _MAX_ROW_BYTES:
-        return _pack_f32(query, False), _pack_f32(key, True)
     return _device_layout(query), _device_layout(key)
 
 
@@ -194,8 +189,7 @@ def flash_colreduce(
     """Per-key sum / mean / max over queries of softmax(Q K^T * scale), shape (B, H, N).
 
     Args follow the reference (flash.py:311-352): query (B,H,M,D), key (B,H,N,D), fp16, bf16 or
-    fp32 on the GPU, D <= 256 (fp32 operands are multiplied in fp32 for D <= 128 and rounded to fp16
-    once above that); `is_causal` applies the right-aligned mask (key j visible to query i iff
+    fp32 on the GPU, D <= 256 (fp32 operands are multiplied in fp32); `is_causal` applies the right-aligned mask (key j visible to query i iff
     j <= i + max(N-M, 0)); `scale` defaults to 1/sqrt(D).
 
     `out_dtype` (keyword only, not in the reference) selects the result dtype.  None reproduces

@@ -12,8 +12,8 @@
  *   - q is [B,H,M,D], k is [B,H,N,D], fp16, bf16 or fp32 elements (dtype below).  Strides are in
  *     ELEMENTS, order (batch, head, row, d); the d stride must be 1, row/head/batch strides must be
  *     multiples of 16 bytes (8 16-bit elements, 4 floats) and the base pointers 16-byte aligned; a row
- *     must be a multiple of 16 bytes and at most 512 bytes long: D a multiple of 8 in [8, 256] for
- *     16-bit elements, a multiple of 4 in [4, 128] for fp32.  Rows must not overlap (row stride >= D).
+ *     must be a multiple of 16 bytes and D at most 256: D a multiple of 8 in [8, 256] for
+ *     16-bit elements, a multiple of 4 in [4, 256] for fp32.  Rows must not overlap (row stride >= D).
  *     (The reference takes any strides, flash.py:292-299; a caller with other layouts makes a
  *     contiguous, zero-padded copy first -- the Python host does.)  fp32 operands are multiplied at
  *     full precision and range (the reference's tl.dot rounds them to TF32, flash.py:59,108).
@@ -47,7 +47,7 @@ extern "C" {
 /* element type of q and k */
 #define FCR_DTYPE_F16 0
 #define FCR_DTYPE_BF16 1
-#define FCR_DTYPE_F32 2 /* fp32 operands on the fp32 matrix instructions: D a multiple of 4, at most 128 */
+#define FCR_DTYPE_F32 2 /* fp32 operands on the fp32 matrix instructions: D a multiple of 4, at most 256 */
 
 /* column reduction over query rows */
 #define FCR_REDUCE_SUM 0 /* also the numerator of 'mean' (flash.py:121-122) */
@@ -57,7 +57,7 @@ extern "C" {
 /* argument errors */
 #define FCR_E_NULL -1      /* a required pointer is NULL */
 #define FCR_E_DTYPE -2     /* dtype is not FCR_DTYPE_* */
-#define FCR_E_SHAPE -3     /* B,H,M,N < 1, a row of D elements not a multiple of 16 bytes in [16,512], sizes overflow */
+#define FCR_E_SHAPE -3     /* B,H,M,N < 1, D > 256 or a row of D elements not a multiple of 16 bytes, sizes overflow */
 #define FCR_E_STRIDE -4    /* d stride != 1 or a stride / base pointer breaks 16-byte alignment */
 #define FCR_E_REDUCTION -5 /* reduction is not FCR_REDUCE_* */
 #define FCR_E_SCALE -6     /* scale is not finite */
@@ -130,8 +130,8 @@ int fcr_topk_mask_ws(const float* scores, uint8_t* mask, float* threshold, int64
                      size_t ws_bytes, void* stream);
 
 /*
- * fp32 operands with D > 128, or as a faster and less exact alternative to FCR_DTYPE_F32 (values must
- * fit fp16): packs a contiguous fp32 [rows, D] into the fp16 [rows, terms * Dp] (Dp = D rounded up
+ * A faster and less exact alternative to FCR_DTYPE_F32 for fp32 operands whose values fit fp16 (the
+ * 16-bit matrix instructions run at 16 times the fp32 rate): packs a contiguous fp32 [rows, D] into the fp16 [rows, terms * Dp] (Dp = D rounded up
  * to 8, zero padded) that the kernels above take with D' = terms * Dp and dtype FCR_DTYPE_F16.
  * terms = 3 writes [hi | hi | lo] for queries (is_key = 0) and [hi | lo | hi] for keys (is_key != 0),
  * hi = fp16(x), lo = fp16(x - hi): the kernels then see q.k to about 2^-22.  terms = 1 writes [hi].

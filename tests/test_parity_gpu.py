@@ -82,29 +82,44 @@ def test_config1_fp32():
 
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("m,n,d", [(100, 260, 20), (257, 300, 80), (64, 500, 128), (300, 300, 100), (33, 700, 6),
-                                   (130, 140, 200)])
+                                   (130, 140, 200), (300, 420, 132), (64, 1000, 256), (257, 129, 252),
+                                   (40, 3000, 160)])
 def test_fp32_operands(m, n, d, causal):
-    """fp32 inputs.  D <= 128: fp32 products (held to 1e-5, which no 16-bit rounding of the operands
-    meets; D = 6 is zero padded to 8).  D in (128, 256]: the operands are rounded to fp16 once, like
-    the TF32 rounding of the reference's tl.dot (flash.py:59,108), and only then is the tolerance
-    looser than the metric's."""
+    """fp32 inputs are multiplied in fp32 for every D up to 256: held to 1e-5, which no 16-bit rounding of
+    the operands meets (D = 6 is zero padded to 8; rows of more than 512 bytes take the 1 KiB ring)."""
     q, k = _inputs.randn_pair(2, 2, m, n, d, seed=d, dtype=torch.float32)
     qd, kd = q.cuda(), k.cuda()
     for red in REDUCTIONS:
         got = fca.flash_colreduce(qd, kd, red, is_causal=causal, scale=0.11)
         want = colreduce_ref(q, k, red, causal, scale=0.11, compute_dtype=torch.float64).float()
         assert got.dtype == torch.float32
-        if d <= 128:
-            check(got, want, red, f"fp32 d{d}")
-            torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-8)
-        else:
-            torch.testing.assert_close(got.cpu(), want, rtol=5e-3, atol=1e-5)
+        check(got, want, red, f"fp32 d{d}")
+        torch.testing.assert_close(got.cpu(), want, rtol=1e-5, atol=1e-8)
 
 
-def test_fp32_operands_beyond_the_fp16_range():
+@pytest.mark.parametrize("terms,d,rtol", [(3, 80, 2e-5), (3, 20, 2e-5), (1, 200, 5e-3)])
+def test_fp32_operands_packed_for_the_16_bit_matrix_instructions(terms, d, rtol):
+    """fcr_pack_f32 + FCR_DTYPE_F16 through the C ABI: the faster, less exact way to feed fp32 operands
+    (three fp16 segments give products to about 2^-22, one segment is a single rounding to fp16)."""
+    from flash_colreduce_amd import _lib, flash as F
+    b, h, m, n = 2, 2, 130, 700
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=terms + d, dtype=torch.float32)
+    qp, kp = F.pack_f32(q.cuda(), False, terms), F.pack_f32(k.cuda(), True, terms)
+    lib = _lib.load()
+    out = torch.empty(b * h, n, device="cuda")
+    lse = torch.empty(lib.fcr_lse_bytes(b, h, m, n, qp.shape[3]) // 4, device="cuda")
+    _lib.check(lib.fcr_colreduce(qp.data_ptr(), kp.data_ptr(), out.data_ptr(), lse.data_ptr(), _lib.DTYPE_F16, b, h, m, n,
+                                 qp.shape[3], _lib.strides4(qp.stride()), _lib.strides4(kp.stride()), 0.11,
+                                 _lib.REDUCE_SUM, 1, torch.cuda.current_stream().cuda_stream))
+    want = colreduce_ref(q, k, "sum", True, scale=0.11, compute_dtype=torch.float64).float()
+    torch.testing.assert_close(out.view(b, h, n).cpu(), want, rtol=rtol, atol=1e-7)
+
+
+@pytest.mark.parametrize("d", [64, 192])
+def test_fp32_operands_beyond_the_fp16_range(d):
     """fp32 keeps its range: queries of magnitude 3e5 (an fp16 rounding would give inf and NaN results)
     with a scale that brings the scores back to order one, and keys of magnitude 1e-7."""
-    b, h, m, n, d = 1, 3, 200, 333, 64
+    b, h, m, n = 1, 3, 200, 333
     q, k = _inputs.randn_pair(b, h, m, n, d, seed=77, dtype=torch.float32)
     for fq, fk in ((3e5, 1.0), (1.0, 1e-7), (2e4, 2e4)):
         qq, kk = q * fq, k * fk
