@@ -17,11 +17,13 @@ SRC = os.path.join(HERE, "csrc", "fcr.hip")
 INCLUDE = os.path.join(ROOT, "include")
 LIB = os.path.join(HERE, "libfcr.so")
 
+OBJ_DIR = os.path.join(HERE, "_build")
+PARTS = (0, 1, 2, 3, 4)   # -DFCR_PART=n, see the top of csrc/fcr.hip
+
 HIPCC_FLAGS = [
     "-O3",
     "--offload-arch=gfx950",
     "-std=c++17",
-    "-shared",
     "-fPIC",
     "-fno-gpu-rdc",
     # keep packed fp32 VALU forms out of the generated code
@@ -37,10 +39,25 @@ def hipcc_path() -> str:
 
 
 def build(verbose: bool = True, extra_flags=()) -> str:
-    cmd = [hipcc_path(), *HIPCC_FLAGS, *extra_flags, "-I", INCLUDE, SRC, "-o", LIB]
+    """Compiles the parts of csrc/fcr.hip side by side (one hipcc each) and links them into libfcr.so."""
+    hipcc = hipcc_path()
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    jobs = []
+    for part in PARTS:
+        obj = os.path.join(OBJ_DIR, f"fcr_part{part}.o")
+        # a part uses a subset of the file's helpers
+        cmd = [hipcc, *HIPCC_FLAGS, *extra_flags, f"-DFCR_PART={part}", "-Wno-unused-function", "-I", INCLUDE,
+               "-c", SRC, "-o", obj]
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        jobs.append((cmd, obj, subprocess.Popen(cmd)))
+    failed = [cmd for cmd, _, proc in jobs if proc.wait() != 0]
+    if failed:
+        raise subprocess.CalledProcessError(1, failed[0])
+    link = [hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *[obj for _, obj, _ in jobs], "-o", LIB]
     if verbose:
-        print(" ".join(cmd), flush=True)
-    subprocess.run(cmd, check=True)
+        print(" ".join(link), flush=True)
+    subprocess.run(link, check=True)
     return LIB
 
 

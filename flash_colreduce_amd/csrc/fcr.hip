@@ -36,7 +36,48 @@
 
 #include "fcr.h"
 
+// The file can be compiled whole, or in parts that are linked together (the build script does that to
+// use several cores): part 0 holds the C ABI and the small kernels, parts 1-4 the sweeps of one element
+// type each (fp16, bf16, fp32 rows up to 512 bytes, longer fp32 rows).
+#ifndef FCR_PART
+#define FCR_PART -1
+#endif
+#define FCR_HAS(part) (FCR_PART == -1 || FCR_PART == (part))
+
+namespace fcr_detail {
+struct Params {
+  const char* q;
+  const char* k;
+  float* lse;        // [BH, M]
+  float* part;       // [splits, BH, M] partial lse of key ranges when splits > 1
+  int splits;        // key ranges per row tile in the row kernel (1 = whole sweep in one workgroup)
+  void* out;         // [BH, N]: column sums or means (or the only result)
+  void* out2;        // [BH, N]: column maxima when one sweep produces both
+  int64_t q_sb, q_sh, q_sr;  // strides in BYTES: batch, head, row
+  int64_t k_sb, k_sh, k_sr;
+  int H, M, N;
+  int dgran;         // D / 8: valid 16-byte granules per row
+  int c;             // max(N - M, 0): the causal right-alignment offset
+  float scale2;      // scale * log2(e)
+  int tiles;         // resident tiles per (b,h)
+  int bh_count;      // B * H
+  int group;         // (b,h) pairs whose workgroups are launched together (see map_block)
+  int stream_once;   // col_small_kernel: load the keys non-temporally
+  int total;         // tiles * B * H workgroups
+  // How the column kernels write a finished column (see store_column)
+  int out_fmt;       // element type of out and out2: FCR_DTYPE_F32, FCR_DTYPE_F16 or FCR_DTYPE_BF16
+  int mean_from;     // < 0: out holds the sums.  Else out holds means: columns below mean_from are
+  float inv_m;       //   multiplied by inv_m = 1/M, column j from there on is divided by N - j
+};
+// which: 0 = row statistics, 1 = column sweep, 2 = column sweep for few queries (16-bit types only)
+void sweeps_f16(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
+void sweeps_bf16(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
+void sweeps_f32(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
+void sweeps_f32_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
+}  // namespace fcr_detail
+
 namespace {
+using fcr_detail::Params;
 
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -100,30 +141,6 @@ constexpr int kChunk = 64;                    // streamed rows per LDS stage (tw
 constexpr float kNegInf = -__builtin_inff();
 constexpr float kPosInf = __builtin_inff();
 
-struct Params {
-  const char* q;
-  const char* k;
-  float* lse;        // [BH, M]
-  float* part;       // [splits, BH, M] partial lse of key ranges when splits > 1
-  int splits;        // key ranges per row tile in the row kernel (1 = whole sweep in one workgroup)
-  void* out;         // [BH, N]: column sums or means (or the only result)
-  void* out2;        // [BH, N]: column maxima when one sweep produces both
-  int64_t q_sb, q_sh, q_sr;  // strides in BYTES: batch, head, row
-  int64_t k_sb, k_sh, k_sr;
-  int H, M, N;
-  int dgran;         // D / 8: valid 16-byte granules per row
-  int c;             // max(N - M, 0): the causal right-alignment offset
-  float scale2;      // scale * log2(e)
-  int tiles;         // resident tiles per (b,h)
-  int bh_count;      // B * H
-  int group;         // (b,h) pairs whose workgroups are launched together (see map_block)
-  int stream_once;   // col_small_kernel: load the keys non-temporally
-  int total;         // tiles * B * H workgroups
-  // How the column kernels write a finished column (see store_column)
-  int out_fmt;       // element type of out and out2: FCR_DTYPE_F32, FCR_DTYPE_F16 or FCR_DTYPE_BF16
-  int mean_from;     // < 0: out holds the sums.  Else out holds means: columns below mean_from are
-  float inv_m;       //   multiplied by inv_m = 1/M, column j from there on is divided by N - j
-};
 
 // D[16 keys][16 queries] += A[16 keys][32 d] * B[32 d][16 queries].  Lane l supplies, for A and for
 // B alike, the 8 consecutive d-elements [8*(l/16), +8) of row / column l & 15, and receives
@@ -1690,8 +1707,8 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
     default: CALL(DT, 8); break;                           \
   }
 
-// fp32 rows are twice as long: up to 16 k-steps
-#define FCR_DISPATCH_KS_F32(ksteps, CALL)                         \
+// fp32 rows of more than 512 bytes: 9 to 16 k-steps
+#define FCR_DISPATCH_KS_F32_LONG(ksteps, CALL)                    \
   switch (ksteps) {                                               \
     case 9: CALL(FCR_DTYPE_F32, 9); break;                        \
     case 10: CALL(FCR_DTYPE_F32, 10); break;                      \
@@ -1700,8 +1717,7 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
     case 13: CALL(FCR_DTYPE_F32, 13); break;                      \
     case 14: CALL(FCR_DTYPE_F32, 14); break;                      \
     case 15: CALL(FCR_DTYPE_F32, 15); break;                      \
-    case 16: CALL(FCR_DTYPE_F32, 16); break;                      \
-    default: FCR_DISPATCH_KS(FCR_DTYPE_F32, ksteps, CALL)         \
+    default: CALL(FCR_DTYPE_F32, 16); break;                      \
   }
 
 #define FCR_DISPATCH_KS4(DT, ksteps, CALL)                 \
@@ -1714,7 +1730,48 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
 
 }  // namespace
 
+// The sweeps of one element type (see the declarations at the top).
+#define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal, s)
+#define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal, mode, s)
+#define FCR_CALL_COL_SMALL(DT, KS) launch_col_small<DT, KS>(p, causal, mode, s)
+#define FCR_SWEEPS_16BIT(NAME, DT)                                                                       \
+  void fcr_detail::NAME(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) { \
+    if (which == 0) { FCR_DISPATCH_KS(DT, ksteps, FCR_CALL_LSE) }                                        \
+    else if (which == 1) { FCR_DISPATCH_KS(DT, ksteps, FCR_CALL_COL) }                                   \
+    else { FCR_DISPATCH_KS4(DT, ksteps, FCR_CALL_COL_SMALL) }                                            \
+  }
+#if FCR_HAS(1)
+FCR_SWEEPS_16BIT(sweeps_f16, FCR_DTYPE_F16)
+#endif
+#if FCR_HAS(2)
+FCR_SWEEPS_16BIT(sweeps_bf16, FCR_DTYPE_BF16)
+#endif
+#if FCR_HAS(3)
+void fcr_detail::sweeps_f32(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
+  if (which == 0) { FCR_DISPATCH_KS(FCR_DTYPE_F32, ksteps, FCR_CALL_LSE) }
+  else { FCR_DISPATCH_KS(FCR_DTYPE_F32, ksteps, FCR_CALL_COL) }
+}
+#endif
+#if FCR_HAS(4)
+void fcr_detail::sweeps_f32_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
+  if (which == 0) { FCR_DISPATCH_KS_F32_LONG(ksteps, FCR_CALL_LSE) }
+  else { FCR_DISPATCH_KS_F32_LONG(ksteps, FCR_CALL_COL) }
+}
+#endif
+#undef FCR_CALL_LSE
+#undef FCR_CALL_COL
+#undef FCR_CALL_COL_SMALL
+
+#if FCR_HAS(0)
 namespace {
+// sweeps of the element type `dtype`
+void launch_sweeps(int dtype, int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
+  if (dtype == FCR_DTYPE_F16) fcr_detail::sweeps_f16(which, p, ksteps, causal, mode, s);
+  else if (dtype == FCR_DTYPE_BF16) fcr_detail::sweeps_bf16(which, p, ksteps, causal, mode, s);
+  else if (ksteps <= kMaxKSteps) fcr_detail::sweeps_f32(which, p, ksteps, causal, mode, s);
+  else fcr_detail::sweeps_f32_long_rows(which, p, ksteps, causal, mode, s);
+}
+
 template <int VPT>
 void launch_topk_spread(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, uint32_t* w,
                         hipStream_t s) {
@@ -1761,11 +1818,7 @@ int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int 
   p.group = head_group(p.bh_count, (int64_t)p.tiles * p.splits, causal != 0);
   const int ksteps = ksteps_of(dtype, D);
   hipStream_t s = static_cast<hipStream_t>(stream);
-#define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal != 0, s)
-  if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_LSE) }
-  else if (dtype == FCR_DTYPE_BF16) { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_LSE) }
-  else { FCR_DISPATCH_KS_F32(ksteps, FCR_CALL_LSE) }
-#undef FCR_CALL_LSE
+  launch_sweeps(dtype, 0, p, ksteps, causal != 0, 0, s);
   rc = launched("row_lse_kernel");
   if (rc || p.splits == 1) return rc;
   const int64_t rows = (int64_t)B * H * M;
@@ -1819,18 +1872,11 @@ int col_reduce_any(const void* q, const void* k, const float* lse, void* out, vo
       p.total = (int)(p.bh_count * splits);
       p.group = head_group(p.bh_count, splits, false);
       p.stream_once = ((int64_t)p.bh_count * N * p.dgran * 16 >= (1ll << 30)) ? 1 : 0;
-#define FCR_CALL_COL_SMALL(DT, KS) launch_col_small<DT, KS>(p, causal != 0, mode, s)
-      if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS4(FCR_DTYPE_F16, ksteps, FCR_CALL_COL_SMALL) }
-      else { FCR_DISPATCH_KS4(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL_SMALL) }
-#undef FCR_CALL_COL_SMALL
+      launch_sweeps(dtype, 2, p, ksteps, causal != 0, mode, s);
       return launched("col_small_kernel");
     }
   }
-#define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal != 0, mode, s)
-  if (dtype == FCR_DTYPE_F16) { FCR_DISPATCH_KS(FCR_DTYPE_F16, ksteps, FCR_CALL_COL) }
-  else if (dtype == FCR_DTYPE_BF16) { FCR_DISPATCH_KS(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL) }
-  else { FCR_DISPATCH_KS_F32(ksteps, FCR_CALL_COL) }
-#undef FCR_CALL_COL
+  launch_sweeps(dtype, 1, p, ksteps, causal != 0, mode, s);
   return launched("col_reduce_kernel");
 }
 }  // namespace
@@ -1983,3 +2029,4 @@ int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, in
 }
 
 }  // extern "C"
+#endif  // FCR_HAS(0)
