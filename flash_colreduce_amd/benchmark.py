@@ -1,6 +1,6 @@
 """Latency / peak-memory sweep over the reference's 20 benchmark shapes.
 
-    python -m flash_colreduce_amd.benchmark [--budget SECONDS] [--no-naive] [--rows 0,13] [--out FILE]
+    python -m flash_colreduce_amd.benchmark [--budget SECONDS] [--no-naive] [--rows 0,13] [--dtype fp16|bf16|fp32] [--out FILE]
     python -m flash_colreduce_amd.benchmark --topk
 
 Same shapes and method as the reference's harness (benchmarks/run.py:11-92): fp16, H = 32, D = 128,
@@ -57,9 +57,12 @@ def measure_memory(fn) -> float:
     return torch.cuda.max_memory_allocated() / 2**20
 
 
-def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None):
+DTYPES = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}
+
+
+def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None, dtype: str = "fp16"):
     name = torch.cuda.get_device_name(0)
-    print(f"Benchmark results on {name} (fp16, reduction=sum)", file=out)
+    print(f"Benchmark results on {name} ({dtype}, reduction=sum)", file=out)
     head = (f"{'configuration':<48} {'flash ms':>10} {'naive ms':>10} {'speedup':>8} {'flash MB':>10} "
             f"{'naive MB':>10} {'mem saving':>10} {'TFLOP/s':>9}")
     print(head, file=out)
@@ -71,8 +74,8 @@ def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None)
                 continue
             b, h, m, n, d, causal = (cfg[k] for k in ("b", "h", "m", "n", "d", "is_causal"))
             g = torch.Generator(device="cuda").manual_seed(0)
-            q = torch.randn(b, h, m, d, device="cuda", dtype=torch.float16, generator=g)
-            k = torch.randn(b, h, n, d, device="cuda", dtype=torch.float16, generator=g)
+            q = torch.randn(b, h, m, d, device="cuda", dtype=DTYPES[dtype], generator=g)
+            k = torch.randn(b, h, n, d, device="cuda", dtype=DTYPES[dtype], generator=g)
             flash = lambda: flash_colreduce(q, k, reduction="sum", is_causal=causal)  # noqa: E731
             naive = lambda: naive_colreduce(q, k, reduction="sum", is_causal=causal)  # noqa: E731
             f_ms, f_mb = measure_latency(flash, budget), measure_memory(flash)
@@ -135,6 +138,7 @@ def main():
     ap.add_argument("--no-naive", action="store_true", help="skip the materialising implementation")
     ap.add_argument("--rows", default=None, help="comma separated indices (0..19) of the shapes to run; default all")
     ap.add_argument("--out", default=None, help="also write the table to this file")
+    ap.add_argument("--dtype", default="fp16", choices=sorted(DTYPES), help="element type of q and k (the reference's table is fp16)")
     ap.add_argument("--topk", action="store_true", help="time the top-k keep-mask against torch.topk instead")
     args = ap.parse_args()
     if not torch.cuda.is_available():
@@ -145,10 +149,10 @@ def main():
     only = None if args.rows is None else {int(r) for r in args.rows.split(",")}
     if args.out:
         with open(args.out, "w") as f:
-            run(args.budget, not args.no_naive, out=f, only=only)
+            run(args.budget, not args.no_naive, out=f, only=only, dtype=args.dtype)
         print(open(args.out).read())
     else:
-        run(args.budget, not args.no_naive, only=only)
+        run(args.budget, not args.no_naive, only=only, dtype=args.dtype)
 
 
 if __name__ == "__main__":
