@@ -124,16 +124,19 @@ inline int64_t rows_swept(int M, int nb) {
 // One block also wins when two would give between one and two workgroups per CU (with fewer than
 // one the keys of a tile are split over workgroups instead, see row_splits; that case does not depend
 // on `causal`, so the size of the lse buffer does not either).  With the mask exactly two per CU is
-// still too coarse: the chip then waits for the workgroup with the longest sweep.
-inline int row_blocks_per_wave(int ksteps, int M, int64_t bh, bool causal) {
+// still too coarse: the chip then waits for the workgroup with the longest sweep.  Against at most
+// 1024 keys one block wins below one workgroup per CU as well: twice the workgroups beat splitting
+// sweeps of 16 chunks (32 heads of 1024 x 1024: 16.5 -> 14 us, 16 heads of 512 x 512: 13 -> 8.6 us).
+inline int row_blocks_per_wave(int ksteps, int M, int N, int64_t bh, bool causal) {
   if (ksteps > 4) return 1;
   if (rows_swept(M, 1) * (100 + 3 * ksteps) < rows_swept(M, 2) * 100) return 1;
   const int64_t wgs2 = bh * ((M + kWaves * 64 - 1) / (kWaves * 64));
   const int cus = chip_cus();
+  if (wgs2 < cus && N <= 1024) return 1;
   return (wgs2 >= cus && wgs2 < 2 * cus + (causal ? 1 : 0)) ? 1 : 2;
 }
-inline int row_tile_rows(int ksteps, int M, int64_t bh, bool causal) {
-  return kWaves * 32 * row_blocks_per_wave(ksteps, M, bh, causal);
+inline int row_tile_rows(int ksteps, int M, int N, int64_t bh, bool causal) {
+  return kWaves * 32 * row_blocks_per_wave(ksteps, M, N, bh, causal);
 }
 constexpr int kMaxKSteps = 8;                 // 16-bit elements: D <= 256
 constexpr int kMaxKStepsF32 = 16;             // fp32: D <= 256 as well (rows of up to 1 KiB, one workgroup per CU)
@@ -771,7 +774,9 @@ inline int col_tile_blocks(int ksteps, int mode, int N, int64_t bh, bool causal)
   const int cus = chip_cus();
   // two-block tiles only when they still give two workgroups per CU; with fewer, CUs idle or run a single
   // workgroup (32 heads of 1024 x 1024: the call takes 37 us with 128 two-block tiles, 32 us with 256 one-block tiles)
+  // (without the mask one workgroup on most CUs does better with two blocks: 16 heads of 4096 x 4096 76 -> 66 us)
   if (causal) return wgs2 <= 2 * cus ? 1 : 2;
+  if (wgs2 <= cus) return 2 * wgs2 > cus ? 2 : 1;
   return wgs2 < 2 * cus ? 1 : 2;
 }
 
@@ -1588,7 +1593,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   if (rc) return rc;
   // the device is first asked (for its CU count) here, after every argument check
   const int ksteps = ksteps_of(dtype, D);
-  const int trows = by_keys ? kWaves * 32 * col_tile_blocks(ksteps, col_mode, N, bh, causal) : row_tile_rows(ksteps, M, bh, causal);
+  const int trows = by_keys ? kWaves * 32 * col_tile_blocks(ksteps, col_mode, N, bh, causal) : row_tile_rows(ksteps, M, N, bh, causal);
   const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
   p.q = static_cast<const char*>(q);
   p.k = static_cast<const char*>(k);
@@ -1617,7 +1622,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
 // workgroup per CU; otherwise the keys of a tile are split so that about two per CU run, each
 // keeping at least four 64-key chunks.
 int row_splits(int B, int H, int M, int N, int ksteps) {
-  const int trows = row_tile_rows(ksteps, M, (int64_t)B * H, false);  // same with the mask when wgs < 256
+  const int trows = row_tile_rows(ksteps, M, N, (int64_t)B * H, false);  // same with the mask when wgs < 256
   const int64_t wgs = (int64_t)B * H * ((M + trows - 1) / trows);
   const int64_t chunks = (N + kChunk - 1) / kChunk;
   const int cus = chip_cus();
@@ -1645,7 +1650,7 @@ void launch_lse_blocks(const Params& p, bool causal, hipStream_t s) {
 template <int DT, int KS>
 void launch_lse(const Params& p, bool causal, hipStream_t s) {
   if constexpr (KS <= 4) {
-    if (row_blocks_per_wave(KS, p.M, p.bh_count, causal) == 2) return launch_lse_blocks<DT, KS, 2, false>(p, causal, s);
+    if (row_blocks_per_wave(KS, p.M, p.N, p.bh_count, causal) == 2) return launch_lse_blocks<DT, KS, 2, false>(p, causal, s);
   }
   // one row tile per (b,h) and at least 1 GiB of keys: stream them past the caches
   const int64_t key_bytes = (int64_t)p.bh_count * p.N * p.dgran * 16;
