@@ -676,6 +676,13 @@ __global__ __launch_bounds__(kThreads, (KS > 8 ? 1 : 2)) void row_lse_kernel(con
     for (int sub = 0; sub < kChunk / 32; ++sub) {
       const int key0 = t * kChunk + sub * 32;
       if (key0 >= p.N) continue;
+      // the sub-step's fragments once, for all groups that see it
+      u32x4 kf[2][KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        kf[0][ks] = rg.frag(lds, sub, 0, ks);
+        kf[1][ks] = rg.frag(lds, sub, 1, ks);
+      }
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
         const int qg = q0[g];
@@ -683,8 +690,8 @@ __global__ __launch_bounds__(kThreads, (KS > 8 ? 1 : 2)) void row_lse_kernel(con
         f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          acc[0] = mma<DT>(rg.frag(lds, sub, 0, ks), qf[g][ks], acc[0]);
-          acc[1] = mma<DT>(rg.frag(lds, sub, 1, ks), qf[g][ks], acc[1]);
+          acc[0] = mma<DT>(kf[0][ks], qf[g][ks], acc[0]);
+          acc[1] = mma<DT>(kf[1][ks], qf[g][ks], acc[1]);
         }
         const bool need_mask = (key0 + 32 > p.N) || (CAUSAL && key0 + 31 > qg + p.c);
         if (need_mask) lse_update<true>(acc, p.scale2, mref[g], l[g], last[g] - key0);
@@ -859,6 +866,13 @@ __global__ __launch_bounds__(kThreads, ((NB > 2 || KS > 8) ? 1 : 2)) void col_re
       // +inf for rows past M: they contribute 2^-inf = 0
       if (qs + (lane & 15) >= p.M) lq.v[0] = kPosInf;
       if (qs + 16 + (lane & 15) >= p.M) lq.v[1] = kPosInf;
+      // the sub-step's fragments once, for all groups that see it
+      u32x4 qfrag[2][KS];
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        qfrag[0][ks] = rg.frag(lds, sub, 0, ks);
+        qfrag[1][ks] = rg.frag(lds, sub, 1, ks);
+      }
 #pragma unroll
       for (int g = 0; g < NG; ++g) {
         const int kg = k0[g];
@@ -867,8 +881,8 @@ __global__ __launch_bounds__(kThreads, ((NB > 2 || KS > 8) ? 1 : 2)) void col_re
         f32x4 acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-          acc[0] = mma<DT>(kf[g][ks], rg.frag(lds, sub, 0, ks), acc[0]);
-          acc[1] = mma<DT>(kf[g][ks], rg.frag(lds, sub, 1, ks), acc[1]);
+          acc[0] = mma<DT>(kf[g][ks], qfrag[0][ks], acc[0]);
+          acc[1] = mma<DT>(kf[g][ks], qfrag[1][ks], acc[1]);
         }
         const bool need_mask = CAUSAL && (kg + 15 > qs + p.c);
         if (need_mask) col_update<true, MODE>(acc, p.scale2, lq.v, csum[g], cmax[g], lim_lane + qs - kg);
