@@ -6,6 +6,7 @@ a C ABI (include/fcr.h); torch is used for device memory and the current stream 
 """
 from __future__ import annotations
 
+import functools
 import math
 from typing import Optional
 
@@ -49,6 +50,9 @@ def _device_layout(x: torch.Tensor) -> torch.Tensor:
     """
     d = x.shape[3]
     al = 16 // x.element_size()   # elements per 16 bytes: 8 (fp16, bf16) or 4 (fp32)
+    if (d % al == 0 and x.is_contiguous() and x.data_ptr() % 16 == 0 and x.stride(2) == d and
+            x.stride(0) % al == 0 and x.stride(1) % al == 0):
+        return x   # the usual case (dimensions of size one may carry any stride, hence the last three tests)
     if d % al != 0:
         return torch.nn.functional.pad(x, (0, al - d % al))  # new contiguous tensor
     ok = (x.stride(3) == 1 and x.data_ptr() % 16 == 0 and
@@ -85,6 +89,21 @@ def _operands(query, key):
 _REDUCTIONS = {"sum": _lib.REDUCE_SUM, "max": _lib.REDUCE_MAX, "mean": _lib.REDUCE_MEAN}
 
 
+@functools.lru_cache(maxsize=4096)
+def _lse_floats(dev_index: int, b: int, h: int, m: int, n: int, d: int) -> int:
+    """Floats of the row-statistics buffer (fcr_lse_bytes depends on the device's CU count, hence dev_index)."""
+    with torch.cuda.device(dev_index):
+        return max(b * h * m, _lib.load().fcr_lse_bytes(b, h, m, n, d) // 4)
+
+
+def _raw_stream(dev: torch.device) -> int:
+    """The current stream of `dev` as a hipStream_t value."""
+    try:
+        return torch._C._cuda_getCurrentRawStream(dev.index if dev.index is not None else torch.cuda.current_device())
+    except AttributeError:   # the private shortcut is gone: the public, slower way
+        return torch.cuda.current_stream(dev).cuda_stream
+
+
 def _launch_to(query, key, reduction, is_causal, scale, res_dtype):
     """One reduction, finished on the device: the column kernel stores res_dtype and divides the means
     (fcr_colreduce_to), so nothing is left for torch to do after the two launches.  Needs M, N, B*H > 0."""
@@ -95,13 +114,19 @@ def _launch_to(query, key, reduction, is_causal, scale, res_dtype):
     q, k = _operands(query, key)
     lib = _lib.load()
     dev = query.device
-    lse = torch.empty(max(b * h * m, lib.fcr_lse_bytes(b, h, m, n, q.shape[3]) // 4), device=dev, dtype=torch.float32)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    lse = torch.empty(_lse_floats(index, b, h, m, n, q.shape[3]), device=dev, dtype=torch.float32)
     out = torch.empty((b, h, n), device=dev, dtype=res_dtype)
-    with torch.cuda.device(dev):
-        _lib.check(lib.fcr_colreduce_to(q.data_ptr(), k.data_ptr(), out.data_ptr(), _DTYPES[res_dtype], lse.data_ptr(),
-                                        _DTYPES[q.dtype], b, h, m, n, q.shape[3], _lib.strides4(q.stride()),
-                                        _lib.strides4(k.stride()), float(scale), _REDUCTIONS[reduction],
-                                        int(bool(is_causal)), torch.cuda.current_stream(dev).cuda_stream))
+    args = (q.data_ptr(), k.data_ptr(), out.data_ptr(), _DTYPES[res_dtype], lse.data_ptr(), _DTYPES[q.dtype], b, h, m, n,
+            q.shape[3], _lib.strides4(q.stride()), _lib.strides4(k.stride()), float(scale), _REDUCTIONS[reduction],
+            1 if is_causal else 0)
+    if torch.cuda.current_device() == index:
+        rc = lib.fcr_colreduce_to(*args, _raw_stream(dev))
+    else:
+        with torch.cuda.device(index):
+            rc = lib.fcr_colreduce_to(*args, _raw_stream(dev))
+    if rc:
+        _lib.check(rc)
     return out
 
 
