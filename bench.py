@@ -38,7 +38,7 @@ PEAK_HBM_TBPS = 8.0
 # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # scaled by the same counters on a 256 MiB device copy (FETCH unit 2 KiB, WRITE unit 1 KiB);
 # the summary of those runs is profiles/headline_causal_8192_fp16.md.
-HBM_TRAFFIC_BYTES = {"row_lse_kernel": 218.0e6 + 1.05e6, "col_reduce_kernel": 196.1e6 + 1.05e6}
+HBM_TRAFFIC_BYTES = {"row_lse_kernel": 229.5e6 + 1.05e6, "col_reduce_kernel": 199.7e6 + 1.05e6}
 CONDITIONING_SECONDS = 0.4
 CONFIG_CONDITIONING_SECONDS = 0.25   # per workload and reduction of the configs array, untimed
 
