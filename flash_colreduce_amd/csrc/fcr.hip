@@ -331,14 +331,6 @@ __device__ __forceinline__ void store_column(const Params& p, void* base, bool i
   }
 }
 
-// A store to LDS that the compiler does not see as one: before a store it does see, it waits for
-// every load-to-LDS in flight (they might write the same bytes), which would drain the ring.  The
-// caller keeps the order: a barrier with lgkmcnt(0) stands between this store and any read of it.
-__device__ __forceinline__ void lds_store_unordered(float* slot, float v) {
-  asm volatile("ds_write_b32 %0, %1" ::"v"((uint32_t)(uintptr_t)(__attribute__((address_space(3))) float*)slot), "v"(v)
-               : "memory");
-}
-
 template <int N>
 __device__ __forceinline__ void ring_sync() {
   asm volatile("" ::: "memory");
@@ -1076,12 +1068,12 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
     if (MODE != kModeMax) {
       vsum += __shfl_xor(vsum, 16);
       vsum += __shfl_xor(vsum, 32);
-      if (lane < 16) lds_store_unordered(obuf + slot, vsum);
+      if (lane < 16) obuf[slot] = vsum;
     }
     if (MODE != kModeSum) {
       vmax = fmaxf(vmax, __shfl_xor(vmax, 16));
       vmax = fmaxf(vmax, __shfl_xor(vmax, 32));
-      if (lane < 16) lds_store_unordered(obuf_max + slot, fast_exp2(vmax));
+      if (lane < 16) obuf_max[slot] = fast_exp2(vmax);
     }
   }
   ring_sync<0>();   // the loads past the last chunk write their zeros before the LDS is given back
