@@ -296,21 +296,24 @@ def topk_keep_mask(scores: torch.Tensor, k: int, return_threshold: bool = False)
     """Boolean mask of the k largest entries along the last dimension (ties: lower index wins).
 
     The step a pruning caller takes on the (B, H, N) result of flash_colreduce; not part of the
-    reference's package.  `scores` must be a float32 GPU tensor; the result has its shape.
+    reference's package.  `scores` is a float32, float16 or bfloat16 GPU tensor; the result has its shape.
     With return_threshold also returns the k-th largest value per row, shape scores.shape[:-1].
     """
     if not scores.is_cuda:
         raise ValueError("scores must be on CUDA device.")
-    if scores.dtype != torch.float32 or scores.dim() < 1:
-        raise ValueError(f"scores must be a float32 tensor with at least one dimension. Got {scores.dtype}.")
-    s = scores.contiguous()
+    if scores.dtype not in _DTYPES or scores.dim() < 1:
+        raise ValueError(f"scores must be a float32, float16 or bfloat16 tensor with at least one dimension. "
+                         f"Got {scores.dtype}.")
+    # 16-bit scores (what flash_colreduce returns for 16-bit operands) are widened first: exact, so the
+    # order and the ties are those of the 16-bit values
+    s = scores.contiguous() if scores.dtype == torch.float32 else scores.float().contiguous()
     n = s.shape[-1]
     rows = s.numel() // n if n else 0
     if rows > 0 and n > 0:
         mask = torch.empty(s.shape, device=s.device, dtype=torch.bool)   # the kernel writes every entry
     else:
         mask = torch.zeros(s.shape, device=s.device, dtype=torch.bool)
-    thr = torch.empty(s.shape[:-1], device=s.device, dtype=torch.float32) if return_threshold else None
+    thr = torch.empty(s.shape[:-1], device=s.device, dtype=torch.float32) if return_threshold else None   # always fp32
     if rows > 0 and n > 0:
         lib = _lib.load()
         nbytes = lib.fcr_topk_bytes(rows, n)   # > 0 for long rows: scratch that lets workgroups share a row

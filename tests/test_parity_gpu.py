@@ -596,6 +596,19 @@ def test_topk_long_rows_with_and_without_scratch(rows, n, k):
         assert torch.equal(thr.cpu(), kth), use_ws
 
 
+def test_topk_takes_the_operator_result_as_it_comes():
+    """fp16 / bf16 scores, as flash_colreduce returns them for 16-bit operands: same mask as for their fp32 values."""
+    from oracle.colreduce_oracle import topk_mask_ref
+    q, k = _inputs.randn_pair(1, 3, 200, 3000, 64, seed=21, dtype=torch.bfloat16)
+    scores = fca.flash_colreduce(q.cuda(), k.cuda(), "sum", is_causal=True)
+    assert scores.dtype == torch.bfloat16
+    mask = fca.topk_keep_mask(scores, 500)
+    want = topk_mask_ref(scores.float().cpu().view(3, 3000).numpy(), 500)
+    assert (mask.view(3, 3000).cpu().numpy() == want).all()
+    with pytest.raises(ValueError):
+        fca.topk_keep_mask(scores.to(torch.float64), 5)
+
+
 def test_topk_on_reduced_columns():
     from oracle.colreduce_oracle import topk_mask_ref
     q, k = _inputs.config4(heads=4, n=2048)
