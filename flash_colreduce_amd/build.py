@@ -63,5 +63,22 @@ def build(verbose: bool = True, extra_flags=()) -> str:
     return LIB
 
 
+C_CHECK_SRC = os.path.join(ROOT, "tests", "c_abi", "check.c")
+C_CHECK_BIN = os.path.join(ROOT, "tests", "c_abi", "check")
+
+
+def build_c_check(verbose: bool = True) -> str:
+    """The plain C caller of the library (tests/c_abi/check.c), linked against libfcr.so next to this file.
+    (Compiled as C, where the HIP headers have to be told the platform.)"""
+    cmd = [hipcc_path(), "-x", "c", "-O1", "-D__HIP_PLATFORM_AMD__", "-I", INCLUDE, "-I", "/opt/rocm/include", C_CHECK_SRC,
+           "-o", C_CHECK_BIN, "-L", HERE, "-lfcr", "-L", "/opt/rocm/lib", "-lamdhip64", "-lm",
+           "-Wl,-rpath,$ORIGIN/../../flash_colreduce_amd", "-Wl,-rpath,/opt/rocm/lib"]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    subprocess.run(cmd, check=True)
+    return C_CHECK_BIN
+
+
 if __name__ == "__main__":
     build(extra_flags=sys.argv[1:])
+    build_c_check()

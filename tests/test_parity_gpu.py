@@ -729,6 +729,17 @@ def test_launcher_stub_of_the_integration_notes():
         assert torch.equal(got, fca.flash_colreduce(qd, kd, red, is_causal=causal))
 
 
+def test_plain_c_caller_of_the_c_abi():
+    """tests/c_abi/check.c: hipMalloc, fcr_colreduce, closed forms; no Python or torch in that process."""
+    import os
+    import subprocess
+    from flash_colreduce_amd import build as fcr_build
+    if not os.path.exists(fcr_build.C_CHECK_BIN):
+        fcr_build.build_c_check(verbose=False)
+    done = subprocess.run([fcr_build.C_CHECK_BIN], capture_output=True, text=True, timeout=100)
+    assert done.returncode == 0 and done.stdout.strip() == "ok", (done.returncode, done.stdout, done.stderr)
+
+
 def test_python_errors_on_device():
     q = torch.zeros(1, 2, 4, 8, dtype=torch.float16, device="cuda")
     k = torch.zeros(1, 2, 6, 8, dtype=torch.float16, device="cuda")
