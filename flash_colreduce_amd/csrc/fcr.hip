@@ -141,6 +141,7 @@ inline int row_tile_rows(int ksteps, int M, int N, int64_t bh, bool causal) {
 constexpr int kMaxKSteps = 8;                 // 16-bit elements: D <= 256
 constexpr int kMaxKStepsF32 = 16;             // fp32: D <= 256 as well (rows of up to 1 KiB, one workgroup per CU)
 constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row sub-steps)
+constexpr int64_t kMaxWorkgroups = 1ll << 24; // the runtime refuses launches of 2^32 threads or more
 constexpr float kNegInf = -__builtin_inff();
 constexpr float kPosInf = __builtin_inff();
 
@@ -1542,14 +1543,20 @@ int fail(int code, const char* what) {
 inline int elem_bytes(int dtype) { return dtype == FCR_DTYPE_F32 ? 4 : 2; }
 inline int ksteps_of(int dtype, int D) { return (D * elem_bytes(dtype) + 63) / 64; }
 
-int check_strides(const void* ptr, const int64_t s[4], const char* name, int rows, int D, int esize) {
+// dims = sizes of the batch, head and row dimensions.  The stride of a dimension of size one is never
+// used to form an address, so it may be anything (torch reports arbitrary strides there, and a slice of an
+// expanded tensor keeps stride 0): only the strides that matter are checked.
+int check_strides(const void* ptr, const int64_t s[4], const char* name, const int dims[3], int D, int esize) {
   if (s[3] != 1) {
     snprintf(g_err, sizeof(g_err), "%s: stride of the last dimension must be 1 (got %lld)", name, (long long)s[3]);
     return FCR_E_STRIDE;
   }
   const int al = 16 / esize;   // elements per 16 bytes
-  if ((reinterpret_cast<uintptr_t>(ptr) & 15) != 0 || s[0] % al != 0 || s[1] % al != 0 || s[2] % al != 0 ||
-      s[0] < 0 || s[1] < 0 || s[2] < 0 || s[2] * esize >= (1 << 25)) {
+  bool ok = (reinterpret_cast<uintptr_t>(ptr) & 15) == 0;
+  for (int i = 0; i < 3; ++i)
+    if (dims[i] > 1 && (s[i] % al != 0 || s[i] < 0)) ok = false;
+  if (dims[2] > 1 && s[2] * esize >= (1 << 25)) ok = false;
+  if (!ok) {
     snprintf(g_err, sizeof(g_err),
              "%s: base pointer must be 16-byte aligned, batch/head/row strides non-negative multiples of 16 bytes (%d elements), row stride < 2^25 bytes",
              name, al);
@@ -1557,7 +1564,7 @@ int check_strides(const void* ptr, const int64_t s[4], const char* name, int row
   }
   // Rows that overlap (an expanded operand has row stride 0) cannot be described by the buffer views
   // the kernels read through: the view of the rows from r on is (rows - r) * stride bytes long.
-  if (rows > 1 && s[2] < D) {
+  if (dims[2] > 1 && s[2] < D) {
     snprintf(g_err, sizeof(g_err), "%s: row stride (%lld) must be at least D (%d) when there is more than one row",
              name, (long long)s[2], D);
     return FCR_E_STRIDE;
@@ -1591,11 +1598,14 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
                                          : "D must be a multiple of 4 in [4, 256] for FCR_DTYPE_F32");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
-  if (bh * (((int64_t)(by_keys ? N : M) + 127) / 128) > (1ll << 30)) return fail(FCR_E_SHAPE, "B*H*tiles exceeds 2^30 workgroups");
+  // a launch may have fewer than 2^32 threads: fewer than 2^24 workgroups of 256 (the finest tiling, 128 rows)
+  if (bh * (((int64_t)(by_keys ? N : M) + 127) / 128) >= kMaxWorkgroups)
+    return fail(FCR_E_SHAPE, "B*H*ceil(rows/128) must be below 2^24 workgroups");
   if (!isfinite(scale)) return fail(FCR_E_SCALE, "scale must be finite");
-  int rc = check_strides(q, qs, "q", M, D, esize);
+  const int qdims[3] = {B, H, M}, kdims[3] = {B, H, N};
+  int rc = check_strides(q, qs, "q", qdims, D, esize);
   if (rc) return rc;
-  rc = check_strides(k, ks, "k", N, D, esize);
+  rc = check_strides(k, ks, "k", kdims, D, esize);
   if (rc) return rc;
   // the device is first asked (for its CU count) here, after every argument check
   const int ksteps = ksteps_of(dtype, D);
@@ -1603,8 +1613,9 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   const int64_t tiles = ((by_keys ? N : M) + trows - 1) / trows;
   p.q = static_cast<const char*>(q);
   p.k = static_cast<const char*>(k);
-  p.q_sb = qs[0] * esize; p.q_sh = qs[1] * esize; p.q_sr = qs[2] * esize;
-  p.k_sb = ks[0] * esize; p.k_sh = ks[1] * esize; p.k_sr = ks[2] * esize;
+  // a single row is given the stride of a dense one: the buffer views are sized rows * stride
+  p.q_sb = B > 1 ? qs[0] * esize : 0; p.q_sh = H > 1 ? qs[1] * esize : 0; p.q_sr = M > 1 ? qs[2] * esize : D * esize;
+  p.k_sb = B > 1 ? ks[0] * esize : 0; p.k_sh = H > 1 ? ks[1] * esize : 0; p.k_sr = N > 1 ? ks[2] * esize : D * esize;
   p.H = H; p.M = M; p.N = N;
   p.dgran = D * esize / 16;
   p.c = N > M ? N - M : 0;
@@ -1911,7 +1922,7 @@ int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float
 size_t fcr_topk_bytes(int64_t rows, int N) {
   if (rows < 1 || N <= 32 * kTopkThreads || N > (1 << 30)) return 0;
   const int parts = (N + 8 * kTopkThreads - 1) / (8 * kTopkThreads);   // the finer of the two ways to cut a row
-  if (rows * parts > 0x7fffffffll) return 0;
+  if (rows * parts >= (1ll << 22)) return 0;   // more workgroups of 1024 threads than one launch may have
   return 2 * topk_hist_words(rows, parts) * sizeof(uint32_t) + (size_t)rows * 4 * sizeof(TopkState);
 }
 
@@ -1932,7 +1943,8 @@ int fcr_topk_mask_ws(const float* scores, uint8_t* mask, float* threshold, int64
 
 int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream) {
   if (!scores || !mask) return fail(FCR_E_NULL, "null pointer argument");
-  if (rows < 1 || rows > 0x7fffffffll || N < 1) return fail(FCR_E_SHAPE, "rows must be in [1, 2^31) and N >= 1");
+  // one workgroup of 1024 threads per row, fewer than 2^32 threads per launch
+  if (rows < 1 || rows >= (1ll << 22) || N < 1) return fail(FCR_E_SHAPE, "rows must be in [1, 2^22) and N >= 1");
   const dim3 grid((unsigned)rows), block(kTopkThreads);
   hipStream_t s = static_cast<hipStream_t>(stream);
   if (N <= 8 * kTopkThreads) hipLaunchKernelGGL(topk_mask_kernel<8>, grid, block, 0, s, scores, mask, threshold, N, k);
@@ -2020,7 +2032,8 @@ int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, in
   if (!out) return fail(FCR_E_NULL, "null pointer argument");
   if (reduction != FCR_REDUCE_SUM && reduction != FCR_REDUCE_MAX)
     return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM or FCR_REDUCE_MAX");
-  // every argument check of the two kernels, before the device is asked for anything
+  // every argument check of the two kernels first (the last step of make_params asks the device for its
+  // CU count; nothing else has touched it by then)
   Params p;
   int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, false, causal != 0);
   if (rc) return rc;

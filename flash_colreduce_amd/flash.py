@@ -143,8 +143,8 @@ def _launch(query, key, kinds, is_causal, scale):
     lib = _lib.load()
     dev = query.device
     # the row statistics, followed by whatever scratch the row kernel wants for this shape
-    nfloat = max(b * h * m, lib.fcr_lse_bytes(b, h, m, n, q.shape[3]) // 4)
-    lse = torch.empty(nfloat, device=dev, dtype=torch.float32)
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    lse = torch.empty(_lse_floats(index, b, h, m, n, q.shape[3]), device=dev, dtype=torch.float32)
     outs = [torch.empty((b * h, n), device=dev, dtype=torch.float32) for _ in kinds]
     if b * h * m * n == 0:
         lse.fill_(float("-inf"))

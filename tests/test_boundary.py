@@ -70,7 +70,9 @@ def test_c_abi_rejects_bad_arguments_without_a_device(fn):
         (dict(dtype=2, D=260), -3), (dict(dtype=2, D=6), -3),                 # fp32: a multiple of 4, at most 256
         (dict(dtype=2, D=64, qs=(512, 512, 66, 1)), -4),                       # fp32: strides in multiples of 4
         (dict(qs=(512, 512, 64, 2)), -4), (dict(ks=(512, 512, 60, 1)), -4), (dict(q=18), -4),
-        (dict(ks=(512, -512, 64, 1)), -4),
+        (dict(H=2, ks=(512, -512, 64, 1)), -4), (dict(B=2, qs=(-512, 512, 64, 1)), -4),
+        (dict(H=2, qs=(512, 4, 64, 1)), -4),                                   # head stride not a multiple of 16 bytes
+        (dict(B=1 << 12, H=1 << 12), -3),                                      # 2^24 workgroups: more threads than a launch may have
         (dict(qs=(512, 512, 0, 1)), -4), (dict(ks=(512, 512, 32, 1)), -4),   # overlapping rows
         (dict(scale=float("inf")), -6), (dict(scale=float("nan")), -6),
     ]

@@ -376,6 +376,32 @@ def test_expanded_operands(causal):
 
 
 @pytest.mark.parametrize("causal", [False, True])
+def test_single_row_with_any_row_stride(causal):
+    """One query row or one key row whose row stride is smaller than D (a slice of an expanded tensor keeps
+    stride 0; torch reports arbitrary strides for dimensions of size one): the stride of a single row is
+    never used, through the operator and through the C ABI alike."""
+    from flash_colreduce_amd import _lib
+    b, h, d = 2, 3, 64
+    q, k = _inputs.randn_pair(b, h, 40, 700, d, seed=77)
+    qd, kd = q.cuda(), k.cuda()
+    q1 = qd[:, :, 7:8].expand(b, h, 5, d)[:, :, :1]       # M = 1, row stride 0
+    k1 = kd[:, :, 9:10].expand(b, h, 6, d)[:, :, :1]      # N = 1, row stride 0
+    assert q1.stride(2) == 0 and k1.stride(2) == 0
+    lib = _lib.load()
+    for qx, kx in ((q1, kd), (qd, k1), (q1, k1)):
+        m, n = qx.shape[2], kx.shape[2]
+        for red in REDUCTIONS:
+            got = fca.flash_colreduce(qx, kx, red, is_causal=causal, out_dtype=torch.float32)
+            check(got, colreduce_ref(qx.cpu(), kx.cpu(), red, causal), red, f"m{m} n{n}")
+        out = torch.empty(b * h, n, device="cuda")
+        lse = torch.empty(lib.fcr_lse_bytes(b, h, m, n, d) // 4, device="cuda")
+        _lib.check(lib.fcr_colreduce(qx.data_ptr(), kx.data_ptr(), out.data_ptr(), lse.data_ptr(), _lib.DTYPE_F16, b, h,
+                                     m, n, d, _lib.strides4(qx.stride()), _lib.strides4(kx.stride()), 0.125, 0,
+                                     int(causal), None))
+        check(out.view(b, h, n), colreduce_ref(qx.cpu(), kx.cpu(), "sum", causal), "sum", f"C ABI m{m} n{n}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
 def test_score_jumps_renormalise(causal):
     """Scores that jump by far more than 64 binades in the middle of the sweep, and rows whose
     scores are all hugely negative: exercises the renormalisation of the running row sum."""
@@ -721,12 +747,13 @@ def test_launcher_stub_of_the_integration_notes():
     code = code.replace("/path/to/libfcr.so", _lib.LIB_PATH)
     scope = {}
     exec(compile(code, "INTEGRATION.md", "exec"), scope)
-    q, k = _inputs.randn_pair(2, 3, 130, 1000, 64, seed=4)
-    qd, kd = q.cuda(), k.cuda()
-    for red, causal in (("sum", True), ("max", False)):
-        got = scope["_flash_colreduce"](qd, kd, red, causal, 0.125)
-        assert got.dtype == torch.float16 and got.shape == (2, 3, 1000)
-        assert torch.equal(got, fca.flash_colreduce(qd, kd, red, is_causal=causal))
+    for dtype in (torch.float16, torch.bfloat16, torch.float32):   # the three element types the reference's tl.dot takes
+        q, k = _inputs.randn_pair(2, 3, 130, 1000, 64, seed=4, dtype=dtype)
+        qd, kd = q.cuda(), k.cuda()
+        for red, causal in (("sum", True), ("max", False)):
+            got = scope["_flash_colreduce"](qd, kd, red, causal, 0.125)
+            assert got.dtype == dtype and got.shape == (2, 3, 1000)
+            assert torch.equal(got, fca.flash_colreduce(qd, kd, red, is_causal=causal, scale=0.125))
 
 
 def test_plain_c_caller_of_the_c_abi():
@@ -734,8 +761,11 @@ def test_plain_c_caller_of_the_c_abi():
     import os
     import subprocess
     from flash_colreduce_amd import build as fcr_build
-    if not os.path.exists(fcr_build.C_CHECK_BIN):
-        fcr_build.build_c_check(verbose=False)
+    from flash_colreduce_amd import _lib
+    header = os.path.join(fcr_build.INCLUDE, "fcr.h")
+    newest = max(os.path.getmtime(f) for f in (fcr_build.C_CHECK_SRC, header, _lib.LIB_PATH))
+    if not os.path.exists(fcr_build.C_CHECK_BIN) or os.path.getmtime(fcr_build.C_CHECK_BIN) < newest:
+        fcr_build.build_c_check(verbose=False)   # never a binary older than its source, the header or the library
     done = subprocess.run([fcr_build.C_CHECK_BIN], capture_output=True, text=True, timeout=100)
     assert done.returncode == 0 and done.stdout.strip() == "ok", (done.returncode, done.stdout, done.stderr)
 
