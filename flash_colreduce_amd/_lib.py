@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libfcr.so")
 
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 REDUCE_SUM, REDUCE_MAX, REDUCE_MEAN = 0, 1, 2
+OPT_SINGLE_SWEEP, OPT_WAIT_POLLS = 0, 1
 
 _I64x4 = ctypes.c_int64 * 4
 _lib = None
@@ -64,6 +65,10 @@ def _declare(lib):
     lib.fcr_colreduce_static.restype = c.c_int
     lib.fcr_colreduce_static.argtypes = ([c.c_void_p, c.c_void_p, c.c_void_p] + common +
                                          [c.c_int, c.c_int, c.c_void_p])
+    lib.fcr_set_option.restype = c.c_int
+    lib.fcr_set_option.argtypes = [c.c_int, c.c_longlong]
+    lib.fcr_colreduce_status.restype = c.c_int
+    lib.fcr_colreduce_status.argtypes = [c.c_void_p] + [c.c_int] * 6 + [c.c_void_p]
     return lib
 
 

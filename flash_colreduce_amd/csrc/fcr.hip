@@ -68,12 +68,18 @@ struct Params {
   int out_fmt;       // element type of out and out2: FCR_DTYPE_F32, FCR_DTYPE_F16 or FCR_DTYPE_BF16
   int mean_from;     // < 0: out holds the sums.  Else out holds means: columns below mean_from are
   float inv_m;       //   multiplied by inv_m = 1/M, column j from there on is divided by N - j
+  // col_fused_kernel: teams of `splits` workgroups, team t takes (b,h) = t, t + teams, ..
+  int teams;
+  unsigned* sync;    // arrival counter of team t at sync[32 * t], error word at sync[32 * teams]; all zero at launch
+  int spin_limit;    // polls of the counter after which a wait gives up
 };
-// which: 0 = row statistics, 1 = column sweep, 2 = column sweep for few queries (16-bit types only)
+// which: 0 = row statistics, 1 = column sweep, 2 = column sweep for few queries, 3 = both sweeps in one for few
+// queries, mode + 4 for more than 64 of them (2 and 3: 16-bit types only)
 void sweeps_f16(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_bf16(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_f32(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_f32_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
+extern thread_local bool fused_refused;   // set by a launcher of col_fused_kernel that did not launch
 }  // namespace fcr_detail
 
 namespace {
@@ -402,6 +408,16 @@ struct Ring {
     for (int i = 0; i < kPer; ++i) dma16<AUX>(view, voff[i], stage + (wave * kPer + i) * 1024);
     next_ptr += (int64_t)kChunk * row_bytes32;
     rows_left -= kChunk;
+  }
+  // kChunk rows from `ptr` on into `stage`, of which the first `rows` (clamped to [0, kChunk]) exist;
+  // for sweeps that do not walk one operand front to back.
+  template <int AUX = 0>
+  __device__ __forceinline__ void issue_at(char* stage, const char* ptr, int rows) {
+    const int live = rows_in_chunk(rows);
+    const __amdgpu_buffer_rsrc_t view = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(ptr), 0, (int)((uint32_t)live * row_bytes32), 0x00020000);
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) dma16<AUX>(view, voff[i], stage + (wave * kPer + i) * 1024);
   }
   // Fragment of the 16-row group sg of sub-step `sub` (32 rows) for k-step ks.
   __device__ __forceinline__ u32x4 frag(const char* stage, int sub, int sg, int ks) const {
@@ -1081,6 +1097,325 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
   flush(c0 + (c1 - c0 - 1) / kFlush * kFlush);
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Both sweeps in one for at most 128 query rows against many keys: the keys are read from memory ONCE.
+// A team of p.splits workgroups shares a (b,h) pair; workgroup s of the team owns the kFusedChunks chunks
+// of 64 keys from chunk s * kFusedChunks on.  Per pair ("item") a workgroup
+//   1. streams its keys through the LDS ring and computes their scores against all queries, wave w taking
+//      keys [16w, 16w+16) of each chunk as in col_small_kernel; the scaled scores STAY IN REGISTERS
+//      (16 per lane and chunk);
+//   2. reduces them to the log-sum-exp of every query row over its own keys (row maximum, then the sum:
+//      the scores are at hand, so no running renormalisation is needed) and publishes the 64 or 128 values;
+//   3. meets the other workgroups of its team on an arrival counter in memory, reads their partial values
+//      and merges them into the rows' lse (every workgroup of the team does this merge for itself);
+//   4. turns its scores into probabilities, reduces them down the rows and stores its columns.
+// More than 64 queries: the workgroup has eight waves and waves 4-7 do the same for queries 64-127; the
+// two halves' column results meet in LDS when they are stored.
+// The grid is teams * splits workgroups and never more than the chip holds at once, so every workgroup of a
+// team is running when its partners wait for it; team t takes pairs t, t + teams, t + 2 teams, ..  The
+// keys of the next pair are already streaming into the ring while a workgroup waits.  A wait is bounded:
+// after p.spin_limit polls the workgroup gives up, sets the error word, stores NaN columns for that pair
+// and goes on, so every workgroup reaches its end whatever happens to the others.
+// Memory traffic between workgroups uses device-scope atomics only (partials: relaxed stores and loads,
+// counter: release add / relaxed polls + acquire fence), partial slots alternate between two sets by the
+// parity of the round: a workgroup can be at most one round ahead of the slowest of its team.
+constexpr int kFusedChunks = 8;
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_row(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+// Sum or maximum over each row of 16 lanes; every lane of the row ends up with the result.
+template <bool MAX>
+__device__ __forceinline__ float row16_reduce(float v) {
+  float o = dpp_row<0xB1>(v);    // quad_perm [1,0,3,2]
+  v = MAX ? fmaxf(v, o) : v + o;
+  o = dpp_row<0x4E>(v);          // quad_perm [2,3,0,1]
+  v = MAX ? fmaxf(v, o) : v + o;
+  o = dpp_row<0x141>(v);         // row_half_mirror
+  v = MAX ? fmaxf(v, o) : v + o;
+  o = dpp_row<0x140>(v);         // row_mirror
+  v = MAX ? fmaxf(v, o) : v + o;
+  return v;
+}
+
+__global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ w, int n) {
+  const int i = (int)blockIdx.x * 256 + (int)threadIdx.x;
+  if (i < n) w[i] = 0u;
+}
+
+template <int DT, int KS, bool CAUSAL, int MODE, int QH>
+__global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Params p) {
+  constexpr int KG = kFusedChunks;
+  constexpr int NS = (QH == 1) ? 4 : 6;          // ring stages: two workgroups of 256 threads or one of 512 per CU
+  using Rg = Ring<KS, NS>;
+  constexpr int kRowsWg = 64 * QH;               // query rows a workgroup holds
+  constexpr int kItemKeys = KG * kChunk;
+  constexpr int kRes = (MODE == kModeBoth) ? 2 : 1;
+  constexpr int kObufFloats = QH * kRes * kItemKeys;
+  constexpr int kRedFloats = kWaves * QH * 64;
+  // one LDS object (see col_small_kernel): ring | finished columns | per-wave row partials | per-row values | flag
+  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes + (kObufFloats + kRedFloats + kRowsWg + 4) * 4];
+  float* const obuf = reinterpret_cast<float*>(smem + Rg::kBytes);
+  float* const red = obuf + kObufFloats;
+  float* const rowv = red + kRedFloats;
+  int* const flag = reinterpret_cast<int*>(rowv + kRowsWg);
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int half = (QH == 1) ? 0 : (wave >> 2);   // which 64 queries
+  const int wq = wave & 3;                        // which 16 keys of a chunk
+  const int S = p.splits, T = p.teams;
+  const int team = (int)blockIdx.x / S, split = (int)blockIdx.x - team * S;
+  const int c0 = split * KG;                      // first chunk of this workgroup's keys
+  const int key0 = c0 * kChunk;
+  const int keys_end = min(p.N, key0 + kItemKeys);
+  const int rounds = (p.bh_count - team + T - 1) / T;
+  const int qrow = 4 * (lane >> 4);
+  unsigned* const counter = p.sync + 32 * team;
+  int spin_limit = p.spin_limit;
+
+  Rg rg;
+  rg.init(p.k_sr, p.dgran, lane, wq);
+  rg.row_bytes32 = (uint32_t)p.k_sr;
+  const bool once = p.stream_once != 0;
+  auto stage_of = [&](int q) { return smem + ((uint32_t)q % NS) * Rg::kStage; };
+  // chunk number q of this workgroup's stream: chunk q % KG of its range of the pair of round q / KG
+  auto issue = [&](int q) {
+    if (QH == 2 && half != 0) return;             // the first four waves do the staging
+    const int it = q / KG, j = q - it * KG;
+    const int bh = team + it * T;
+    const int bhc = min(bh, p.bh_count - 1);
+    const int b = bhc / p.H, h = bhc - b * p.H;
+    const int row = (c0 + j) * kChunk;
+    const char* ptr = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh + (int64_t)row * p.k_sr;
+    const int rows = (bh < p.bh_count) ? keys_end - row : 0;   // past the last pair: zeros, nothing is fetched
+    if (once) rg.template issue_at<kLoadOnce>(stage_of(q), ptr, rows);
+    else rg.template issue_at<0>(stage_of(q), ptr, rows);
+  };
+#pragma unroll
+  for (int i = 0; i < NS - 1; ++i) issue(i);
+
+  int qrows[4];
+#pragma unroll
+  for (int g = 0; g < 4; ++g) qrows[g] = 64 * half + 16 * g;
+  u32x4 qf[4][KS];
+  auto load_queries = [&](int bh) {
+    const int b = bh / p.H, h = bh - b * p.H;
+    load_resident<KS, 4>(qf, p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh, p.q_sr, qrows, p.M, p.dgran, lane);
+  };
+  load_queries(team);
+
+  // Register (g, r) of a lane is query 64*half + 16g + qrow + r against the lane's key.  It takes part iff
+  // the query exists and may see the key: 16g + r in [first, mlim).
+  const int mlim = p.M - 64 * half - qrow;
+  const bool ragged_rows = p.M < 64 * (half + 1);
+
+  for (int it = 0; it < rounds; ++it) {
+    const int bh = team + it * T;
+    f32x4 sc[KG][4];
+    // 1. scores of this workgroup's keys, scaled, hidden ones at -inf
+#pragma unroll
+    for (int j = 0; j < KG; ++j) {
+      const int q = it * KG + j;
+      ring_sync<(NS - 2) * Rg::kPer>();   // chunk q visible, the stage of chunk q - 1 is free
+      issue(q + NS - 1);
+      const char* lds = stage_of(q);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) sc[j][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const u32x4 kfrag = rg.frag(lds, wq >> 1, wq & 1, ks);
+#pragma unroll
+        for (int g = 0; g < 4; ++g) sc[j][g] = mma<DT>(qf[g][ks], kfrag, sc[j][g]);
+      }
+      const int kbase = (c0 + j) * kChunk;
+      const int key = kbase + 16 * wq + (lane & 15);
+      const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * half);
+      if (need_mask) {
+        int first = CAUSAL ? key - p.c - 64 * half - qrow : -(1 << 30);
+        if (key >= p.N) first = 1 << 30;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int o = 16 * g + r;
+            sc[j][g][r] = (o >= first && o < mlim) ? sc[j][g][r] * p.scale2 : kNegInf;
+          }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) sc[j][g] *= p.scale2;
+      }
+    }
+    // the queries of the next pair, while this one is finished from the registers
+    if (it + 1 < rounds) load_queries(bh + T);
+
+    // 2. log-sum-exp of every row over this workgroup's keys
+    f32x4 rm[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      rm[g] = sc[0][g];
+#pragma unroll
+      for (int j = 1; j < KG; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) rm[g][r] = fmaxf(rm[g][r], sc[j][g][r]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) rm[g][r] = row16_reduce<true>(rm[g][r]);
+      if ((lane & 15) == 0) *reinterpret_cast<f32x4*>(red + wave * 64 + 16 * g + qrow) = rm[g];
+    }
+    __syncthreads();
+    float my_max = kNegInf;   // of row tid, for tid < kRowsWg
+    if (tid < kRowsWg) {
+      const float* src = red + (tid >> 6) * (kWaves * 64) + (tid & 63);
+      my_max = fmaxf(fmaxf(src[0], src[64]), fmaxf(src[128], src[192]));
+      rowv[tid] = (my_max == kNegInf) ? 0.f : my_max;   // no visible key: any finite reference
+    }
+    __syncthreads();
+    f32x4 rs[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const f32x4 ref = *reinterpret_cast<const f32x4*>(rowv + 64 * half + 16 * g + qrow);
+      rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int j = 0; j < KG; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) rs[g][r] += fast_exp2(sc[j][g][r] - ref[r]);
+#pragma unroll
+      for (int r = 0; r < 4; ++r) rs[g][r] = row16_reduce<false>(rs[g][r]);
+      if ((lane & 15) == 0) *reinterpret_cast<f32x4*>(red + wave * 64 + 16 * g + qrow) = rs[g];
+    }
+    __syncthreads();
+    float* const slots = p.part + ((int64_t)(team * 2 + (it & 1)) * S) * kRowsWg;
+    if (tid < kRowsWg) {
+      const float* src = red + (tid >> 6) * (kWaves * 64) + (tid & 63);
+      const float l = (src[0] + src[64]) + (src[128] + src[192]);
+      // a +inf score makes inf - inf above, a NaN score stays: both give a NaN here, as the row kernel does
+      const float v = (my_max == kNegInf) ? kNegInf : my_max + fast_log2(l);
+      __hip_atomic_store(slots + (int64_t)split * kRowsWg + tid, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();   // every partial of this workgroup has been written
+
+    // 3. meet the team
+    if (tid == 0) {
+      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      const unsigned want = (unsigned)S * (unsigned)(it + 1);
+      int polls = 0, ok = 1;
+      while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
+        if (++polls > spin_limit) {
+          ok = 0;
+          break;
+        }
+        __builtin_amdgcn_s_sleep(4);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      if (!ok) {
+        __hip_atomic_store(p.sync + 32 * T, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        spin_limit = min(spin_limit, 64);   // the call has failed: later waits of this workgroup are short
+      }
+      *flag = ok;
+    }
+    __syncthreads();
+    const bool met = *flag != 0;
+    if (tid < kRowsWg) {
+      float m = kNegInf, acc = 0.f;
+      bool nan = false;
+      for (int s0 = 0; s0 < S; s0 += 8) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+          v[i] = (s0 + i < S) ? __hip_atomic_load(slots + (int64_t)(s0 + i) * kRowsWg + tid, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT)
+                              : kNegInf;
+        float bm = v[0];
+#pragma unroll
+        for (int i = 1; i < 8; ++i) bm = fmaxf(bm, v[i]);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) nan = nan || (v[i] != v[i]);
+        const float nm = fmaxf(m, bm);
+        if (nm > kNegInf) {
+          acc *= fast_exp2(m - nm);
+#pragma unroll
+          for (int i = 0; i < 8; ++i) acc += fast_exp2(v[i] - nm);
+          m = nm;
+        }
+      }
+      const float lse = nan ? __builtin_nanf("") : ((m > kNegInf) ? m + fast_log2(acc) : kNegInf);
+      rowv[tid] = -lse;
+      if (split == 0 && tid < p.M && met) p.lse[(int64_t)bh * p.M + tid] = lse;
+    }
+    __syncthreads();
+
+    // 4. probabilities, reduced down the rows
+    f32x4 nl[4];
+#pragma unroll
+    for (int g = 0; g < 4; ++g) nl[g] = *reinterpret_cast<const f32x4*>(rowv + 64 * half + 16 * g + qrow);
+    float* const osum = obuf + half * (kRes * kItemKeys);
+    float* const omax = osum + (MODE == kModeBoth ? kItemKeys : 0);
+#pragma unroll
+    for (int j = 0; j < KG; ++j) {
+      const int kbase = (c0 + j) * kChunk;
+      const int key = kbase + 16 * wq + (lane & 15);
+      const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * half);
+      float vsum = 0.f, vmax = kNegInf;
+      if (need_mask) {   // hidden entries stay hidden from a row whose lse is not a number
+        int first = CAUSAL ? key - p.c - 64 * half - qrow : -(1 << 30);
+        if (key >= p.N) first = 1 << 30;
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int o = 16 * g + r;
+            const float x = (o >= first && o < mlim) ? sc[j][g][r] + nl[g][r] : kNegInf;
+            if (MODE != kModeSum) vmax = fmaxf(vmax, x);
+            if (MODE != kModeMax) vsum += fast_exp2(x);
+          }
+      } else {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const float x = sc[j][g][r] + nl[g][r];
+            if (MODE != kModeSum) vmax = fmaxf(vmax, x);
+            if (MODE != kModeMax) vsum += fast_exp2(x);
+          }
+      }
+      // the four lane groups hold different queries of the same key
+      const int slot = j * kChunk + 16 * wq + lane;
+      if (MODE != kModeMax) {
+        vsum += __shfl_xor(vsum, 16);
+        vsum += __shfl_xor(vsum, 32);
+        if (lane < 16) osum[slot] = vsum;
+      }
+      if (MODE != kModeSum) {
+        vmax = fmaxf(vmax, __shfl_xor(vmax, 16));
+        vmax = fmaxf(vmax, __shfl_xor(vmax, 32));
+        if (lane < 16) omax[slot] = fast_exp2(vmax);
+      }
+    }
+    __syncthreads();
+    void* const out_max = (MODE == kModeBoth) ? p.out2 : p.out;
+    const float poison = __builtin_nanf("");
+    for (int i = tid; i < kItemKeys; i += kThreads * QH) {
+      if (key0 + i < keys_end) {
+        if (MODE != kModeMax) {
+          float v = obuf[i];
+          if (QH == 2) v += obuf[kRes * kItemKeys + i];
+          store_column(p, p.out, true, bh, key0 + i, met ? v : poison);
+        }
+        if (MODE != kModeSum) {
+          const float* om = obuf + (MODE == kModeBoth ? kItemKeys : 0);
+          float v = om[i];
+          if (QH == 2) v = fmaxf(v, om[kRes * kItemKeys + i]);
+          store_column(p, out_max, false, bh, key0 + i, met ? v : poison);
+        }
+      }
+    }
+    // the next writers of obuf, red, rowv and flag are behind the ring barriers of the next pair
+  }
+  ring_sync<0>();   // the loads past the last chunk write their zeros before the LDS is given back
+}
+
 // ---------------------------------------------------------------------------------------------
 // fp32 operands.  x = hi + lo with hi = fp16(x), lo = fp16(x - hi) carries 22 bits of x.  Packing
 // queries as [hi | hi | lo] and keys as [hi | lo | hi] along d makes the fp16 kernels compute
@@ -1632,6 +1967,9 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   p.out_fmt = FCR_DTYPE_F32;
   p.mean_from = -1;
   p.inv_m = 0.f;
+  p.teams = 0;
+  p.sync = nullptr;
+  p.spin_limit = 0;
   return 0;
 }
 
@@ -1648,6 +1986,33 @@ int row_splits(int B, int H, int M, int N, int ksteps) {
   if (s > chunks / 4) s = chunks / 4;
   if (s > 64) s = 64;
   return s < 1 ? 1 : (int)s;
+}
+
+// The single-sweep path (col_fused_kernel): 16-bit operands, rows of at most 256 bytes, at most 128 queries
+// and enough keys for the sweep to matter.  A (b,h) pair is shared by `splits` workgroups of kFusedChunks
+// chunks each; teams * splits workgroups are launched, never more than the chip holds at once.
+constexpr int kFusedMinChunks = 16;   // 1024 keys
+struct FusedPlan {
+  int qh;       // 1: 64 query rows per workgroup (256 threads, two per CU), 2: 128 (512 threads, one per CU)
+  int splits, teams;
+  int64_t part_at, sync_at;   // where the partial row values and the counters start in the workspace, in floats
+  int64_t floats;             // workspace size
+};
+// Shape conditions only: the size of the workspace must not depend on the element type.
+bool fused_shape(int64_t bh, int M, int N, FusedPlan& f) {
+  const int64_t nchunks = ((int64_t)N + kChunk - 1) / kChunk;
+  if (M > 2 * 64 || nchunks < kFusedMinChunks) return false;
+  f.qh = M > 64 ? 2 : 1;
+  const int cap = chip_cus() * (3 - f.qh);
+  const int64_t splits = (nchunks + kFusedChunks - 1) / kFusedChunks;
+  if (splits > cap) return false;
+  f.splits = (int)splits;
+  const int64_t teams = cap / splits;
+  f.teams = (int)(teams < bh ? teams : bh);
+  f.part_at = (bh * M + 63) / 64 * 64;
+  f.sync_at = f.part_at + 2ll * cap * 64 * f.qh;   // two sets of one slot of 64 * qh values per workgroup
+  f.floats = f.sync_at + ((int64_t)cap + 1) * 32;
+  return true;
 }
 
 int launched(const char* what) {
@@ -1710,6 +2075,50 @@ void launch_col_small(const Params& p, bool causal, int mode, hipStream_t s) {
   else launch_col_small_mode<DT, KS, kModeBoth>(p, causal, s);
 }
 
+// Workgroups of col_fused_kernel wait for each other, so all of a launch must be on the chip together: the
+// host plans with two workgroups of 256 threads, or one of 512, per CU, and the launch is refused (the caller
+// then takes the two-kernel path) if the runtime says that this build of the kernel does not fit that way.
+template <class K>
+bool fits_per_cu(K kernel, int threads, int want) {
+  int n = 0;
+  if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, threads, 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return n >= want;
+}
+
+template <int DT, int KS, int MODE, int QH>
+void launch_col_fused_mode(const Params& p, bool causal, hipStream_t s) {
+  const dim3 grid(p.total), block(kThreads * QH);
+  static int fits[2] = {-1, -1};   // asked once per kernel (the answer depends on its registers and LDS, not on the device of a kind)
+  int f = __atomic_load_n(&fits[causal], __ATOMIC_RELAXED);
+  if (f < 0) {
+    f = causal ? fits_per_cu(col_fused_kernel<DT, KS, true, MODE, QH>, kThreads * QH, 3 - QH)
+               : fits_per_cu(col_fused_kernel<DT, KS, false, MODE, QH>, kThreads * QH, 3 - QH);
+    __atomic_store_n(&fits[causal], f, __ATOMIC_RELAXED);
+  }
+  if (!f) {
+    fcr_detail::fused_refused = true;
+    return;
+  }
+  if (causal) hipLaunchKernelGGL((col_fused_kernel<DT, KS, true, MODE, QH>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((col_fused_kernel<DT, KS, false, MODE, QH>), grid, block, 0, s, p);
+}
+
+// mode: kModeSum or kModeMax, + 4 for the eight-wave form (more than 64 queries)
+template <int DT, int KS>
+void launch_col_fused(const Params& p, bool causal, int mode, hipStream_t s) {
+  const int m = mode & 3;
+  if (mode & 4) {
+    if (m == kModeSum) launch_col_fused_mode<DT, KS, kModeSum, 2>(p, causal, s);
+    else launch_col_fused_mode<DT, KS, kModeMax, 2>(p, causal, s);
+  } else {
+    if (m == kModeSum) launch_col_fused_mode<DT, KS, kModeSum, 1>(p, causal, s);
+    else launch_col_fused_mode<DT, KS, kModeMax, 1>(p, causal, s);
+  }
+}
+
 template <int DT, int KS>
 void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
   if (mode == kModeSum) launch_col_mode<DT, KS, kModeSum>(p, causal, s);
@@ -1756,11 +2165,13 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
 #define FCR_CALL_LSE(DT, KS) launch_lse<DT, KS>(p, causal, s)
 #define FCR_CALL_COL(DT, KS) launch_col<DT, KS>(p, causal, mode, s)
 #define FCR_CALL_COL_SMALL(DT, KS) launch_col_small<DT, KS>(p, causal, mode, s)
+#define FCR_CALL_COL_FUSED(DT, KS) launch_col_fused<DT, KS>(p, causal, mode, s)
 #define FCR_SWEEPS_16BIT(NAME, DT)                                                                       \
   void fcr_detail::NAME(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) { \
     if (which == 0) { FCR_DISPATCH_KS(DT, ksteps, FCR_CALL_LSE) }                                        \
     else if (which == 1) { FCR_DISPATCH_KS(DT, ksteps, FCR_CALL_COL) }                                   \
-    else { FCR_DISPATCH_KS4(DT, ksteps, FCR_CALL_COL_SMALL) }                                            \
+    else if (which == 2) { FCR_DISPATCH_KS4(DT, ksteps, FCR_CALL_COL_SMALL) }                            \
+    else { FCR_DISPATCH_KS4(DT, ksteps, FCR_CALL_COL_FUSED) }                                            \
   }
 #if FCR_HAS(1)
 FCR_SWEEPS_16BIT(sweeps_f16, FCR_DTYPE_F16)
@@ -1783,11 +2194,15 @@ void fcr_detail::sweeps_f32_long_rows(int which, const Params& p, int ksteps, bo
 #undef FCR_CALL_LSE
 #undef FCR_CALL_COL
 #undef FCR_CALL_COL_SMALL
+#undef FCR_CALL_COL_FUSED
 
 #if FCR_HAS(0)
 namespace {
 // sweeps of the element type `dtype`
-void launch_sweeps(int dtype, int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
+void launch_sweeps(int dtype, int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s,
+                   unsigned* zero = nullptr, int zero_words = 0) {
+  if (zero_words > 0)
+    hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((zero_words + 255) / 256)), dim3(256), 0, s, zero, zero_words);
   if (dtype == FCR_DTYPE_F16) fcr_detail::sweeps_f16(which, p, ksteps, causal, mode, s);
   else if (dtype == FCR_DTYPE_BF16) fcr_detail::sweeps_bf16(which, p, ksteps, causal, mode, s);
   else if (ksteps <= kMaxKSteps) fcr_detail::sweeps_f32(which, p, ksteps, causal, mode, s);
@@ -1807,14 +2222,8 @@ void launch_topk_spread(const float* scores, uint8_t* mask, float* threshold, in
 }
 }  // namespace
 
-extern "C" {
-
-int fcr_version(void) { return FCR_VERSION; }
-
-const char* fcr_last_error(void) { return g_err; }
-
-size_t fcr_lse_bytes(int B, int H, int M, int N, int D) {
-  if (B < 1 || H < 1 || M < 1 || N < 1 || D < 1) return 0;
+namespace {
+size_t fcr_lse_bytes_two_kernels(int B, int H, int M, int N) {
   // the most any row width asks for (the tile height, hence the split count, depends a little on the
   // number of 64-byte k-steps of a row), so the size holds for every dtype and D
   int splits = 1;
@@ -1824,6 +2233,32 @@ size_t fcr_lse_bytes(int B, int H, int M, int N, int D) {
   }
   const size_t rows = (size_t)B * (size_t)H * (size_t)M;
   return rows * sizeof(float) * (splits > 1 ? 1 + (size_t)splits : 1);
+}
+
+// process-wide switches (fcr_set_option)
+int g_single_sweep = 1;
+long long g_wait_polls = 1ll << 20;
+}  // namespace
+thread_local bool fcr_detail::fused_refused = false;
+
+extern "C" {
+
+int fcr_version(void) { return FCR_VERSION; }
+
+const char* fcr_last_error(void) { return g_err; }
+
+size_t fcr_lse_bytes(int B, int H, int M, int N, int D) {
+  if (B < 1 || H < 1 || M < 1 || N < 1 || D < 1) return 0;
+  {
+    // the single-sweep path keeps partial row values and its counters behind the row statistics
+    FusedPlan f;
+    if (fused_shape((int64_t)B * H, M, N, f)) {
+      const size_t two_kernels = fcr_lse_bytes_two_kernels(B, H, M, N);
+      const size_t one = (size_t)f.floats * sizeof(float);
+      return one > two_kernels ? one : two_kernels;
+    }
+  }
+  return fcr_lse_bytes_two_kernels(B, H, M, N);
 }
 
 int fcr_row_lse(const void* q, const void* k, float* lse, int dtype, int B, int H, int M, int N, int D,
@@ -1967,22 +2402,61 @@ int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, in
   return launched("pack_f32_kernel");
 }
 
+namespace {
+// Both sweeps of a call, writing `out` in its final form.  ws_bytes = bytes the caller's workspace is known
+// to have (0: what fcr_lse_bytes asks for).  Few queries against many keys take the single sweep.
+int whole_call(const void* q, const void* k, void* out, const ResultSpec& res, float* ws, size_t ws_bytes, int dtype,
+               int B, int H, int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
+               int mode, int causal, void* stream) {
+  Params p;
+  int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true, causal != 0, mode);
+  if (rc) return rc;
+  const int ksteps = ksteps_of(dtype, D);
+  FusedPlan f;
+  if (__atomic_load_n(&g_single_sweep, __ATOMIC_RELAXED) && dtype != FCR_DTYPE_F32 && ksteps <= 4 &&
+      fused_shape(p.bh_count, M, N, f) && (ws_bytes == 0 || (size_t)f.floats * sizeof(float) <= ws_bytes)) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    p.lse = ws;
+    p.part = ws + f.part_at;
+    p.sync = reinterpret_cast<unsigned*>(ws + f.sync_at);
+    p.splits = f.splits;
+    p.teams = f.teams;
+    p.total = f.teams * f.splits;
+    const long long polls = __atomic_load_n(&g_wait_polls, __ATOMIC_RELAXED);
+    p.spin_limit = polls > 0x7fffffffll ? 0x7fffffff : (int)polls;
+    p.out = out;
+    p.out_fmt = res.fmt;
+    if (res.mean) {
+      p.mean_from = causal ? p.c : N;
+      p.inv_m = 1.0f / (float)M;
+    }
+    p.stream_once = ((int64_t)p.bh_count * N * p.dgran * 16 >= (1ll << 30)) ? 1 : 0;
+    const int words = (f.teams + 1) * 32;   // the teams' counters and the error word start at zero
+    fcr_detail::fused_refused = false;
+    launch_sweeps(dtype, 3, p, ksteps, causal != 0, mode | (f.qh == 2 ? 4 : 0), s, p.sync, words);
+    if (!fcr_detail::fused_refused) return launched("col_fused_kernel");
+  }
+  rc = fcr_row_lse(q, k, ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream);
+  if (rc) return rc;
+  return col_reduce_any(q, k, ws, out, nullptr, mode, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream,
+                        res);
+}
+}  // namespace
+
 int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H, int M,
                   int N, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
                   int reduction, int causal, void* stream) {
   if (!out || !lse_ws) return fail(FCR_E_NULL, "null pointer argument");
   if (reduction != FCR_REDUCE_SUM && reduction != FCR_REDUCE_MAX)
     return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM or FCR_REDUCE_MAX");
-  int rc = fcr_row_lse(q, k, lse_ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream);
-  if (rc) return rc;
-  return fcr_col_reduce(q, k, lse_ws, out, dtype, B, H, M, N, D, q_strides, k_strides, scale, reduction,
-                        causal, stream);
+  return whole_call(q, k, out, ResultSpec(), lse_ws, 0, dtype, B, H, M, N, D, q_strides, k_strides, scale,
+                    reduction == FCR_REDUCE_MAX ? kModeMax : kModeSum, causal, stream);
 }
 
 // Scratch of fcr_colreduce_static: the row statistics and, for few query rows against many keys, the
-// partial results of the split row sweep.  One copy per GPU, held until the process ends.  Host code
-// must not pass the array's name to a kernel (it is a host-side stand-in there): the device address is
-// asked once per device and kept.
+// partial results of the split row sweep or the single sweep's partial values and counters.  One copy per
+// GPU, held until the process ends.  Host code must not pass the array's name to a kernel (it is a
+// host-side stand-in there): the device address is asked once per device and kept.
 static __device__ __align__(256) unsigned char scratch[FCR_STATIC_SCRATCH_BYTES];
 
 namespace {
@@ -2017,13 +2491,11 @@ int fcr_colreduce_to(const void* q, const void* k, void* out, int out_dtype, flo
     return fail(FCR_E_REDUCTION, "reduction must be FCR_REDUCE_SUM, FCR_REDUCE_MAX or FCR_REDUCE_MEAN");
   if (out_dtype != FCR_DTYPE_F16 && out_dtype != FCR_DTYPE_BF16 && out_dtype != FCR_DTYPE_F32)
     return fail(FCR_E_DTYPE, "out_dtype must be FCR_DTYPE_F16, FCR_DTYPE_BF16 or FCR_DTYPE_F32");
-  int rc = fcr_row_lse(q, k, lse_ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream);
-  if (rc) return rc;
   ResultSpec res;
   res.fmt = out_dtype;
   res.mean = reduction == FCR_REDUCE_MEAN;
-  return col_reduce_any(q, k, lse_ws, out, nullptr, reduction == FCR_REDUCE_MAX ? kModeMax : kModeSum, dtype, B, H, M,
-                        N, D, q_strides, k_strides, scale, causal, stream, res);
+  return whole_call(q, k, out, res, lse_ws, 0, dtype, B, H, M, N, D, q_strides, k_strides, scale,
+                    reduction == FCR_REDUCE_MAX ? kModeMax : kModeSum, causal, stream);
 }
 
 int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, int B, int H, int M, int N, int D,
@@ -2048,8 +2520,40 @@ int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, in
   float* ws = nullptr;
   rc = static_scratch(&ws);
   if (rc) return rc;
-  // Both kernels write every value of the buffer they later read, so nothing has to be cleared.
+  // The kernels write every value of the buffer they later read (the single sweep's counters are cleared by
+  // a small kernel in front of it), so nothing has to be cleared here.
   return fcr_colreduce(q, k, out, ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, reduction, causal, stream);
+}
+
+int fcr_set_option(int option, long long value) {
+  if (option == FCR_OPT_SINGLE_SWEEP) {
+    __atomic_store_n(&g_single_sweep, value != 0 ? 1 : 0, __ATOMIC_RELAXED);
+    return 0;
+  }
+  if (option == FCR_OPT_WAIT_POLLS) {
+    if (value < 0) return fail(FCR_E_SHAPE, "FCR_OPT_WAIT_POLLS must be >= 0");
+    __atomic_store_n(&g_wait_polls, value, __ATOMIC_RELAXED);
+    return 0;
+  }
+  return fail(FCR_E_SHAPE, "unknown option");
+}
+
+int fcr_colreduce_status(const float* lse_ws, int dtype, int B, int H, int M, int N, int D, void* stream) {
+  if (!lse_ws) return fail(FCR_E_NULL, "null pointer argument");
+  if (B < 1 || H < 1 || M < 1 || N < 1 || D < 1) return fail(FCR_E_SHAPE, "B, H, M, N, D must be >= 1");
+  FusedPlan f;
+  if (dtype == FCR_DTYPE_F32 || ksteps_of(dtype, D) > 4 || !fused_shape((int64_t)B * H, M, N, f)) return 0;
+  unsigned word = 0;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipError_t e = hipMemcpyAsync(&word, reinterpret_cast<const unsigned*>(lse_ws + f.sync_at) + 32 * f.teams,
+                                sizeof(word), hipMemcpyDeviceToHost, s);
+  if (e == hipSuccess) e = hipStreamSynchronize(s);
+  if (e != hipSuccess) {
+    snprintf(g_err, sizeof(g_err), "reading the status word failed: %s", hipGetErrorString(e));
+    return (int)e;
+  }
+  if (word != 0) return fail(FCR_E_WAIT, "a workgroup of the single sweep gave up waiting for its team; the columns of that (b,h) pair are NaN");
+  return 0;
 }
 
 }  // extern "C"

@@ -29,8 +29,9 @@
  *   - Return value: 0 on success; negative FCR_E_* for a rejected argument (nothing was
  *     launched); positive = the hipError_t of a failed launch.  fcr_last_error() returns a
  *     thread-local, human readable description of the last non-zero return on this thread.
- *   - Thread safety: no mutable global state except the thread-local error text; calls from
- *     several threads or streams do not interfere.
+ *   - Thread safety: no mutable global state except the thread-local error text and the switches of
+ *     fcr_set_option; calls from several threads or streams do not interfere (each call needs its own
+ *     lse / workspace buffer while it runs).
  */
 #ifndef FCR_H
 #define FCR_H
@@ -42,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FCR_VERSION 300 /* major*10000 + minor*100 + patch */
+#define FCR_VERSION 310 /* major*10000 + minor*100 + patch */
 
 /* element type of q and k */
 #define FCR_DTYPE_F16 0
@@ -62,6 +63,11 @@ extern "C" {
 #define FCR_E_REDUCTION -5 /* reduction is not FCR_REDUCE_* */
 #define FCR_E_SCALE -6     /* scale is not finite */
 #define FCR_E_SCRATCH -7   /* fcr_colreduce_static: the problem needs more than FCR_STATIC_SCRATCH_BYTES */
+#define FCR_E_WAIT -8      /* fcr_colreduce_status: a workgroup of the single sweep gave up waiting for its team */
+
+/* fcr_set_option */
+#define FCR_OPT_SINGLE_SWEEP 0 /* 0: few queries against many keys take the two kernels as well (default 1) */
+#define FCR_OPT_WAIT_POLLS 1   /* polls of a team's arrival counter after which a workgroup gives up (default 2^20) */
 
 /* size of the built-in scratch buffer of fcr_colreduce_static, per GPU */
 #define FCR_STATIC_SCRATCH_BYTES (16u << 20)
@@ -180,6 +186,25 @@ int fcr_colreduce_to(const void* q, const void* k, void* out, int out_dtype, flo
 int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, int B, int H, int M, int N,
                          int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
                          int reduction, int causal, void* stream);
+
+/*
+ * Few queries against many keys (M <= 128, N >= 1024, 16-bit elements, rows of at most 256 bytes): the calls
+ * that run both kernels (fcr_colreduce, fcr_colreduce_to, fcr_colreduce_static) then take ONE sweep that
+ * reads the keys once, where the reference's kernel reads them twice (flash.py:209-274).  Its workgroups
+ * share a (b,h) pair and meet on counters in the workspace; a workgroup whose partners do not arrive
+ * within FCR_OPT_WAIT_POLLS polls (only possible when the GPU cannot run the whole launch at once, e.g.
+ * under a CU mask) stores NaN columns for that pair, sets a word in the workspace and goes on.
+ * fcr_colreduce_status waits for the stream and returns FCR_E_WAIT if that happened in the last call that
+ * used lse_ws with these sizes, 0 otherwise (also for problems that do not take the single sweep).
+ * No counterpart in the reference, whose kernel has no cross-program dependencies.
+ */
+int fcr_colreduce_status(const float* lse_ws, int dtype, int B, int H, int M, int N, int D, void* stream);
+
+/*
+ * Process-wide switches (FCR_OPT_*), read by every later call: the single sweep on or off (results agree
+ * to rounding either way) and the bound on its waits.  For tests and comparisons; returns 0 or FCR_E_SHAPE.
+ */
+int fcr_set_option(int option, long long value);
 
 #ifdef __cplusplus
 }
