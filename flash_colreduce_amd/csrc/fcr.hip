@@ -70,8 +70,9 @@ struct Params {
   float inv_m;       //   multiplied by inv_m = 1/M, column j from there on is divided by N - j
   // col_fused_kernel: teams of `splits` workgroups, team t takes (b,h) = t, t + teams, ..
   int teams;
-  unsigned* sync;    // arrival counter of team t at sync[32 * t], error word at sync[32 * teams]; all zero at launch
+  unsigned* sync;    // error word; zero at launch, like the slots at `part`
   int spin_limit;    // polls of the counter after which a wait gives up
+  int stagger;       // > 0: every other team starts this many sleeps late (see col_fused_kernel)
 };
 // which: 0 = row statistics, 1 = column sweep, 2 = column sweep for few queries, 3 = both sweeps in one for few
 // queries, mode + 4 for more than 64 of them (2 and 3: 16-bit types only)
@@ -355,12 +356,13 @@ __device__ __forceinline__ int rows_in_chunk(int rows_left) {
   return live;
 }
 
-template <int KS, int NS = ring_stages(KS)>
+// LW: the waves that issue the loads (their index is what init() takes as wave_id)
+template <int KS, int NS = ring_stages(KS), int LW = kWaves>
 struct Ring {
   static constexpr int kN = NS;
   static constexpr int kPitch = KS <= 1 ? 64 : KS == 2 ? 128 : KS <= 4 ? 256 : KS <= 8 ? 512 : 1024;   // LDS row pitch
   static constexpr int kRowsPerLoad = 1024 / kPitch;                 // rows one wave-wide load covers
-  static constexpr int kPer = kChunk / (kWaves * kRowsPerLoad);     // loads per wave and chunk
+  static constexpr int kPer = kChunk / (LW * kRowsPerLoad);          // loads per loading wave and chunk
   static constexpr int kRows = kChunk * kPitch;                      // bytes of rows in a stage
   static constexpr int kStage = kRows + kChunk * 4;                  // rows + 64 floats
   static constexpr int kBytes = kN * kStage;
@@ -1100,27 +1102,29 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
 
 // ---------------------------------------------------------------------------------------------
 // Both sweeps in one for at most 128 query rows against many keys: the keys are read from memory ONCE.
-// A team of p.splits workgroups shares a (b,h) pair; workgroup s of the team owns the kFusedChunks chunks
-// of 64 keys from chunk s * kFusedChunks on.  Per pair ("item") a workgroup
-//   1. streams its keys through the LDS ring and computes their scores against all queries, wave w taking
-//      keys [16w, 16w+16) of each chunk as in col_small_kernel; the scaled scores STAY IN REGISTERS
-//      (16 per lane and chunk);
-//   2. reduces them to the log-sum-exp of every query row over its own keys (row maximum, then the sum:
-//      the scores are at hand, so no running renormalisation is needed) and publishes the 64 or 128 values;
+// A team of p.splits workgroups shares a (b,h) pair; workgroup s of the team owns kFusedSteps chunks of
+// 64 keys; wave w takes keys [16 (w & 3), +16) of each chunk against 64 queries (as in col_small_kernel).
+// Per pair ("item") a workgroup
+//   1. streams its keys through the LDS ring and computes their scores; the scaled scores STAY IN REGISTERS
+//      (16 per lane and step), and the sums of 2^score per row are taken on the way;
+//   2. turns the sums into the log-sum-exp of every row over its own keys and publishes the 64 or 128 values
+//      (sums that left fp32's comfortable range are redone from the registers the exact way, maximum first);
 //   3. meets the other workgroups of its team on an arrival counter in memory, reads their partial values
 //      and merges them into the rows' lse (every workgroup of the team does this merge for itself);
 //   4. turns its scores into probabilities, reduces them down the rows and stores its columns.
-// More than 64 queries: the workgroup has eight waves and waves 4-7 do the same for queries 64-127; the
-// two halves' column results meet in LDS when they are stored.
 // The grid is teams * splits workgroups and never more than the chip holds at once, so every workgroup of a
-// team is running when its partners wait for it; team t takes pairs t, t + teams, t + 2 teams, ..  The
-// keys of the next pair are already streaming into the ring while a workgroup waits.  A wait is bounded:
-// after p.spin_limit polls the workgroup gives up, sets the error word, stores NaN columns for that pair
-// and goes on, so every workgroup reaches its end whatever happens to the others.
-// Memory traffic between workgroups uses device-scope atomics only (partials: relaxed stores and loads,
-// counter: release add / relaxed polls + acquire fence), partial slots alternate between two sets by the
-// parity of the round: a workgroup can be at most one round ahead of the slowest of its team.
-constexpr int kFusedChunks = 8;
+// team is running when its partners wait for it; team t takes pairs t, t + teams, t + 2 teams, ..  The keys of the next pair
+// stream into the ring while a workgroup does steps 2-4.  A wait is bounded: after p.spin_limit polls the
+// workgroup gives up, sets the error word, stores NaN columns for that pair and goes on, so every
+// workgroup reaches its end whatever happens to the others.
+// The barriers between the steps wait for LDS only, so the keys in flight for the next pair stay in
+// flight.  Traffic between workgroups uses device-scope atomics only (relaxed stores and loads, performed
+// where every workgroup of the device sees them); partial slots alternate between two sets by the parity
+// of the round: a workgroup can be at most one round ahead of the slowest of its team.
+constexpr int kFusedSteps = 8;
+#ifndef FCR_FUSED_DBG
+#define FCR_FUSED_DBG 0
+#endif
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_row(float v) {
@@ -1140,88 +1144,180 @@ __device__ __forceinline__ float row16_reduce(float v) {
   return v;
 }
 
+// All LDS accesses of this wave done, then the workgroup's barrier.  Loads and stores to memory stay in flight.
+__device__ __forceinline__ void lds_barrier() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_waitcnt((15) | (3 << 14) | (7 << 4) | (0 << 8));   // vmcnt(63) expcnt(7) lgkmcnt(0)
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 __global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ w, int n) {
   const int i = (int)blockIdx.x * 256 + (int)threadIdx.x;
   if (i < n) w[i] = 0u;
 }
 
+// kFusedSteps chunks of 64 keys per workgroup and pair.  Up to 64 queries (QH = 1): four waves, two
+// workgroups per CU.  Up to 128 (QH = 2): eight waves, waves 4-7 hold queries 64-127, one workgroup per CU.
+// Waves 0-3 load.
 template <int DT, int KS, bool CAUSAL, int MODE, int QH>
 __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Params p) {
-  constexpr int KG = kFusedChunks;
-  constexpr int NS = (QH == 1) ? 4 : 6;          // ring stages: two workgroups of 256 threads or one of 512 per CU
-  using Rg = Ring<KS, NS>;
+  constexpr int KG = kFusedSteps;
+  constexpr int NS = 4 * QH;                     // ring stages (chunks): 66 KiB per workgroup, or 133
+  using Rg = Ring<KS, NS>;                       // waves 0-3 load, four loads of 1 KiB each per chunk for 256-byte rows
+  constexpr int kNumThreads = kThreads * QH;
   constexpr int kRowsWg = 64 * QH;               // query rows a workgroup holds
   constexpr int kItemKeys = KG * kChunk;
   constexpr int kRes = (MODE == kModeBoth) ? 2 : 1;
   constexpr int kObufFloats = QH * kRes * kItemKeys;
   constexpr int kRedFloats = kWaves * QH * 64;
-  // one LDS object (see col_small_kernel): ring | finished columns | per-wave row partials | per-row values | flag
-  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes + (kObufFloats + kRedFloats + kRowsWg + 4) * 4];
+  constexpr int kMergeWaves = 4;                 // waves per row that share the merge of the team's partial values
+  constexpr int kBatch = 8;                      // slots a lane fetches together: one round trip for teams of up to 32
+  constexpr int kMrgFloats = kMergeWaves * kRowsWg * 2;
+  constexpr int kAhead = NS - 1;                 // chunks in flight in front of the one being computed
+  constexpr int kInFlight = (NS - 2) * Rg::kPer; // loads a loader wave may have outstanding when a step starts
+  // one LDS object (see col_small_kernel): ring | finished columns | per-wave row partials | merge | per-row values | flags
+  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes + (kObufFloats + kRedFloats + kMrgFloats + kRowsWg + 4) * 4];
   float* const obuf = reinterpret_cast<float*>(smem + Rg::kBytes);
   float* const red = obuf + kObufFloats;
-  float* const rowv = red + kRedFloats;
+  float* const mrg = red + kRedFloats;
+  float* const rowv = mrg + kMrgFloats;
   int* const flag = reinterpret_cast<int*>(rowv + kRowsWg);
 
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int half = (QH == 1) ? 0 : (wave >> 2);   // which 64 queries
-  const int wq = wave & 3;                        // which 16 keys of a chunk
+  const int tid0 = threadIdx.x, lane0 = tid0 & 63;   // (the loop over the pairs has its own copies, see there)
+  const int wave = __builtin_amdgcn_readfirstlane(tid0 >> 6);
+  const int qh = (QH == 2) ? (wave >> 2) : 0;    // which 64 queries
+  const int wq = wave & 3;                       // which 16 keys of the chunk
+  const bool loader = (QH == 1) || (wave < 4);
   const int S = p.splits, T = p.teams;
   const int team = (int)blockIdx.x / S, split = (int)blockIdx.x - team * S;
-  const int c0 = split * KG;                      // first chunk of this workgroup's keys
+  const int c0 = split * KG;                     // first chunk of this workgroup's keys
   const int key0 = c0 * kChunk;
   const int keys_end = min(p.N, key0 + kItemKeys);
   const int rounds = (p.bh_count - team + T - 1) / T;
-  const int qrow = 4 * (lane >> 4);
-  unsigned* const counter = p.sync + 32 * team;
+  const int qrow0 = 4 * (lane0 >> 4);
   int spin_limit = p.spin_limit;
+  // flag[0]: a row of this workgroup has a sum that must be redone; flag[1]: the team was met.  Each is
+  // written and read on different sides of a barrier.
+  if (tid0 == 0) flag[0] = 0;
 
   Rg rg;
-  rg.init(p.k_sr, p.dgran, lane, wq);
-  rg.row_bytes32 = (uint32_t)p.k_sr;
+  rg.init(p.k_sr, p.dgran, lane0, 0);   // (for the fragment offsets; the loads are issued below)
   const bool once = p.stream_once != 0;
-  auto stage_of = [&](int q) { return smem + ((uint32_t)q % NS) * Rg::kStage; };
-  // chunk number q of this workgroup's stream: chunk q % KG of its range of the pair of round q / KG
-  auto issue = [&](int q) {
-    if (QH == 2 && half != 0) return;             // the first four waves do the staging
-    const int it = q / KG, j = q - it * KG;
-    const int bh = team + it * T;
+  auto stage_of = [&](int c) { return smem + ((uint32_t)c % NS) * Rg::kStage; };   // NS is a power of two
+  // The loaders walk the workgroup's stream of chunks with a running address: KG chunks of one pair, then
+  // the same range of keys of the next pair of the team.  Chunk number c goes to stage c % NS.
+  const int64_t chunk_bytes = (int64_t)kChunk * p.k_sr;
+  const char* run_ptr = nullptr;
+  int run_rows = 0, run_chunk = 0;
+  auto run_to_pair = [&](int bh) {               // the cursor to the start of this workgroup's keys of pair bh
     const int bhc = min(bh, p.bh_count - 1);
     const int b = bhc / p.H, h = bhc - b * p.H;
-    const int row = (c0 + j) * kChunk;
-    const char* ptr = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh + (int64_t)row * p.k_sr;
-    const int rows = (bh < p.bh_count) ? keys_end - row : 0;   // past the last pair: zeros, nothing is fetched
-    if (once) rg.template issue_at<kLoadOnce>(stage_of(q), ptr, rows);
-    else rg.template issue_at<0>(stage_of(q), ptr, rows);
+    run_ptr = p.k + (int64_t)b * p.k_sb + (int64_t)h * p.k_sh + (int64_t)key0 * p.k_sr;
+    run_rows = (bh < p.bh_count) ? keys_end - key0 : 0;   // past the last pair: zeros, nothing is fetched
   };
+  // Where a lane's 16 bytes of each load come from (see Ring::init).  The swizzle repeats every eight rows,
+  // so the kPer loads of a wave have at most kPat different patterns and the rest follow by adding rows.
+  constexpr int kPat = (Rg::kRowsPerLoad >= 8) ? 1 : 8 / Rg::kRowsPerLoad;
+  const int lw = wave & 3;                         // which of the loading waves
+  uint32_t src_off[kPat];
+  bool src_ok[kPat];
 #pragma unroll
-  for (int i = 0; i < NS - 1; ++i) issue(i);
+  for (int e = 0; e < kPat; ++e) {
+    const int byte = (lw * Rg::kPer + e) * 1024 + lane0 * 16;
+    const int row = byte / Rg::kPitch;
+    const int c = ((byte % Rg::kPitch) / 16) ^ Rg::swz(row);
+    src_ok[e] = c < p.dgran;
+    src_off[e] = (uint32_t)row * (uint32_t)p.k_sr + (uint32_t)c * 16u;
+  }
+  const uint32_t pat_bytes = (uint32_t)(kPat * Rg::kRowsPerLoad) * (uint32_t)p.k_sr;
+  auto issue_step = [&]() {
+    if (!loader) return;
+    char* stage = stage_of(run_chunk);
+    const int live = rows_in_chunk(run_rows);
+    const __amdgpu_buffer_rsrc_t view = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<char*>(run_ptr), 0, (int)((uint32_t)live * (uint32_t)p.k_sr), 0x00020000);
+    uint32_t so[kPat];   // opaque copies: the kPer offsets are made per call, not kept in registers between calls
+#pragma unroll
+    for (int e = 0; e < kPat; ++e) {
+      so[e] = src_off[e];
+      asm volatile("" : "+v"(so[e]));
+    }
+    if (once) {
+#pragma unroll
+      for (int i = 0; i < Rg::kPer; ++i) {
+        const uint32_t off = src_ok[i % kPat] ? so[i % kPat] + (uint32_t)(i / kPat) * pat_bytes : kPastEnd;
+        dma16<kLoadOnce>(view, off, stage + (lw * Rg::kPer + i) * 1024);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < Rg::kPer; ++i) {
+        const uint32_t off = src_ok[i % kPat] ? so[i % kPat] + (uint32_t)(i / kPat) * pat_bytes : kPastEnd;
+        dma16<0>(view, off, stage + (lw * Rg::kPer + i) * 1024);
+      }
+    }
+    run_ptr += chunk_bytes;
+    run_rows -= kChunk;
+    ++run_chunk;
+  };
+  run_to_pair(team);
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i) issue_step();
 
   int qrows[4];
 #pragma unroll
-  for (int g = 0; g < 4; ++g) qrows[g] = 64 * half + 16 * g;
+  for (int g = 0; g < 4; ++g) qrows[g] = 64 * qh + 16 * g;
   u32x4 qf[4][KS];
-  auto load_queries = [&](int bh) {
+  // (like load_resident, but the zero padding of D comes from offsets outside the view instead of a select
+  // on the loaded value: nothing here waits for the data, which is first touched by the next pair's MFMAs)
+  auto load_queries = [&](int bh, int lane) {
     const int b = bh / p.H, h = bh - b * p.H;
-    load_resident<KS, 4>(qf, p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh, p.q_sr, qrows, p.M, p.dgran, lane);
+    const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
+    const uint32_t roff = (uint32_t)(lane & 15) * (uint32_t)p.q_sr;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const __amdgpu_buffer_rsrc_t view = rows_view(qb, p.q_sr, qrows[g], p.M);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int gi = ks * 4 + (lane >> 4);
+        qf[g][ks] = view_load16(view, gi < p.dgran ? roff + (uint32_t)gi * 16u : kPastEnd);
+      }
+    }
   };
-  load_queries(team);
+  load_queries(team, lane0);
 
-  // Register (g, r) of a lane is query 64*half + 16g + qrow + r against the lane's key.  It takes part iff
+  // Register (g, r) of a lane is query 64*qh + 16g + qrow + r against the lane's key.  It takes part iff
   // the query exists and may see the key: 16g + r in [first, mlim).
-  const int mlim = p.M - 64 * half - qrow;
-  const bool ragged_rows = p.M < 64 * (half + 1);
+  const int mlim0 = p.M - 64 * qh - qrow0;
+  const bool ragged_rows = p.M < 64 * (qh + 1);
+  constexpr int kRowWaves = kWaves;   // row tid (tid < kRowsWg) is held by four waves: 0-3, or 4-7 for the rows from 64 on
 
+#if FCR_FUSED_DBG & 16
+  long long* const stamps = reinterpret_cast<long long*>(p.out2);
+#define FCR_STAMP(n) if (stamps != nullptr && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 301) && it < 16) stamps[((blockIdx.x ? 1 : 0) * 16 + it) * 8 + (n)] = (long long)wall_clock64();
+#else
+#define FCR_STAMP(n)
+#endif
   for (int it = 0; it < rounds; ++it) {
     const int bh = team + it * T;
     f32x4 sc[KG][4];
+    f32x4 rs[4];   // per row (register) and key (lane): sum of 2^score over the steps
+#pragma unroll
+    for (int g = 0; g < 4; ++g) rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    {
+    const int tid = tid0, lane = lane0, qrow = qrow0, mlim = mlim0;
+    FCR_STAMP(0)
     // 1. scores of this workgroup's keys, scaled, hidden ones at -inf
+    // (what the mask needs is derived afresh from an opaque copy of c0 here and in step 4: kept across the
+    // steps, or hoisted out of the loop over the pairs, it would cost registers that the scores need)
+    int c0a = c0;
+    asm volatile("" : "+s"(c0a));
 #pragma unroll
     for (int j = 0; j < KG; ++j) {
-      const int q = it * KG + j;
-      ring_sync<(NS - 2) * Rg::kPer>();   // chunk q visible, the stage of chunk q - 1 is free
-      issue(q + NS - 1);
-      const char* lds = stage_of(q);
+      ring_sync<kInFlight>();   // the chunks of this step are visible, the stages of the step before are free
+      if (j + kAhead == KG) run_to_pair(bh + T);   // the chunks from here on belong to the next pair
+      issue_step();
+      const char* lds = stage_of(it * KG + j);
 #pragma unroll
       for (int g = 0; g < 4; ++g) sc[j][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -1230,11 +1326,11 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
 #pragma unroll
         for (int g = 0; g < 4; ++g) sc[j][g] = mma<DT>(qf[g][ks], kfrag, sc[j][g]);
       }
-      const int kbase = (c0 + j) * kChunk;
+      const int kbase = (c0a + j) * kChunk;
       const int key = kbase + 16 * wq + (lane & 15);
-      const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * half);
+      const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * qh);
       if (need_mask) {
-        int first = CAUSAL ? key - p.c - 64 * half - qrow : -(1 << 30);
+        int first = CAUSAL ? key - p.c - 64 * qh - qrow : -(1 << 30);
         if (key >= p.N) first = 1 << 30;
 #pragma unroll
         for (int g = 0; g < 4; ++g)
@@ -1247,119 +1343,194 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
 #pragma unroll
         for (int g = 0; g < 4; ++g) sc[j][g] *= p.scale2;
       }
+#pragma unroll
+      for (int g = 0; g < 4; ++g)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) rs[g][r] += fast_exp2(sc[j][g][r]);
     }
-    // the queries of the next pair, while this one is finished from the registers
-    if (it + 1 < rounds) load_queries(bh + T);
+    FCR_STAMP(1)
+    }
+    // From here to the end of the pair, everything that depends on the thread is derived afresh from an
+    // opaque copy of its number: values kept for these steps across step 1 would take registers from the
+    // scores (and come back from scratch memory, a round trip each).
+    int tid_again = threadIdx.x;
+    asm volatile("" : "+v"(tid_again));
+    const int tid = tid_again, lane = tid & 63, qrow = 4 * (lane >> 4);
+    const int mlim = p.M - 64 * qh - qrow;
+    const float* const red_row = red + (tid >> 6) * (kWaves * 64) + (tid & 63);
 
-    // 2. log-sum-exp of every row over this workgroup's keys
-    f32x4 rm[4];
+    // 2. log-sum-exp of every row over this workgroup's keys.  The sums of 2^x were taken as the scores
+    // came; they are good unless a sum left fp32's comfortable range (or a row saw no key at all), and then
+    // the scores, still in registers, are reduced again the exact way: row maximum first.
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
-      rm[g] = sc[0][g];
-#pragma unroll
-      for (int j = 1; j < KG; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) rm[g][r] = fmaxf(rm[g][r], sc[j][g][r]);
-#pragma unroll
-      for (int r = 0; r < 4; ++r) rm[g][r] = row16_reduce<true>(rm[g][r]);
-      if ((lane & 15) == 0) *reinterpret_cast<f32x4*>(red + wave * 64 + 16 * g + qrow) = rm[g];
-    }
-    __syncthreads();
-    float my_max = kNegInf;   // of row tid, for tid < kRowsWg
-    if (tid < kRowsWg) {
-      const float* src = red + (tid >> 6) * (kWaves * 64) + (tid & 63);
-      my_max = fmaxf(fmaxf(src[0], src[64]), fmaxf(src[128], src[192]));
-      rowv[tid] = (my_max == kNegInf) ? 0.f : my_max;   // no visible key: any finite reference
-    }
-    __syncthreads();
-    f32x4 rs[4];
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const f32x4 ref = *reinterpret_cast<const f32x4*>(rowv + 64 * half + 16 * g + qrow);
-      rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int j = 0; j < KG; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) rs[g][r] += fast_exp2(sc[j][g][r] - ref[r]);
 #pragma unroll
       for (int r = 0; r < 4; ++r) rs[g][r] = row16_reduce<false>(rs[g][r]);
       if ((lane & 15) == 0) *reinterpret_cast<f32x4*>(red + wave * 64 + 16 * g + qrow) = rs[g];
     }
-    __syncthreads();
-    float* const slots = p.part + ((int64_t)(team * 2 + (it & 1)) * S) * kRowsWg;
+    lds_barrier();
+    float my_lse = kNegInf;   // of row tid over this workgroup's keys, for tid < kRowsWg
     if (tid < kRowsWg) {
-      const float* src = red + (tid >> 6) * (kWaves * 64) + (tid & 63);
-      const float l = (src[0] + src[64]) + (src[128] + src[192]);
-      // a +inf score makes inf - inf above, a NaN score stays: both give a NaN here, as the row kernel does
-      const float v = (my_max == kNegInf) ? kNegInf : my_max + fast_log2(l);
-      __hip_atomic_store(slots + (int64_t)split * kRowsWg + tid, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();   // every partial of this workgroup has been written
-
-    // 3. meet the team
-    if (tid == 0) {
-      __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-      const unsigned want = (unsigned)S * (unsigned)(it + 1);
-      int polls = 0, ok = 1;
-      while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < want) {
-        if (++polls > spin_limit) {
-          ok = 0;
-          break;
-        }
-        __builtin_amdgcn_s_sleep(4);
-      }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-      if (!ok) {
-        __hip_atomic_store(p.sync + 32 * T, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        spin_limit = min(spin_limit, 64);   // the call has failed: later waits of this workgroup are short
-      }
-      *flag = ok;
-    }
-    __syncthreads();
-    const bool met = *flag != 0;
-    if (tid < kRowsWg) {
-      float m = kNegInf, acc = 0.f;
-      bool nan = false;
-      for (int s0 = 0; s0 < S; s0 += 8) {
-        float v[8];
+      float l = 0.f;
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-          v[i] = (s0 + i < S) ? __hip_atomic_load(slots + (int64_t)(s0 + i) * kRowsWg + tid, __ATOMIC_RELAXED,
-                                                  __HIP_MEMORY_SCOPE_AGENT)
-                              : kNegInf;
+      for (int w = 0; w < kRowWaves; ++w) l += red_row[64 * w];
+      my_lse = fast_log2(l);
+      const bool good = (l >= 8.6736174e-19f) && (l < kPosInf);   // 2^-60: flushed terms are far below the sum's last bit
+      if (!good && tid < p.M) flag[0] = 1;   // (written by whoever finds a bad row; thread 0 resets it below)
+      if (tid == 0) flag[1] = 1;
+    }
+    lds_barrier();
+    if (flag[0] != 0) {   // uniform over the workgroup
+      f32x4 rm[4];
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        rm[g] = sc[0][g];
+#pragma unroll
+        for (int j = 1; j < KG; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) rm[g][r] = fmaxf(rm[g][r], sc[j][g][r]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) rm[g][r] = row16_reduce<true>(rm[g][r]);
+        if ((lane & 15) == 0) *reinterpret_cast<f32x4*>(red + wave * 64 + 16 * g + qrow) = rm[g];
+      }
+      lds_barrier();
+      float my_max = kNegInf;
+      if (tid < kRowsWg) {
+#pragma unroll
+        for (int w = 0; w < kRowWaves; ++w) my_max = fmaxf(my_max, red_row[64 * w]);
+        rowv[tid] = (my_max == kNegInf) ? 0.f : my_max;   // no visible key: any finite reference
+      }
+      lds_barrier();
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4 ref = *reinterpret_cast<const f32x4*>(rowv + 64 * qh + 16 * g + qrow);
+        rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < KG; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) rs[g][r] += fast_exp2(sc[j][g][r] - ref[r]);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) rs[g][r] = row16_reduce<false>(rs[g][r]);
+        if ((lane & 15) == 0) *reinterpret_cast<f32x4*>(red + wave * 64 + 16 * g + qrow) = rs[g];
+      }
+      lds_barrier();
+      if (tid < kRowsWg) {
+        float l = 0.f;
+#pragma unroll
+        for (int w = 0; w < kRowWaves; ++w) l += red_row[64 * w];
+        // a +inf score makes inf - inf above, a NaN score stays: both give a NaN here, as the row kernel does
+        my_lse = (my_max == kNegInf) ? kNegInf : my_max + fast_log2(l);
+      }
+    }
+    // 3. meet the team.  A partial value and the number of its round travel as ONE 64-bit word, so a word
+    // that carries this round's number carries this round's value: nobody waits for a store to complete
+    // and there is no counter.  The slots start at zero (round numbers start at 1).
+    unsigned long long* const slots =
+        reinterpret_cast<unsigned long long*>(p.part) + ((int64_t)(team * 2 + (it & 1)) * S) * kRowsWg;
+    const unsigned round_no = (unsigned)it + 1u;
+    if (tid < kRowsWg)
+      __hip_atomic_store(slots + (int64_t)split * kRowsWg + tid,
+                         ((unsigned long long)round_no << 32) | __builtin_bit_cast(unsigned, my_lse), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    FCR_STAMP(2)
+    // All waves share the team's slots: lane = row, the waves of a row take every kMergeWaves-th slot, poll
+    // until it carries this round, and fold the values into (max, sum).  (The keys a wave has in flight
+    // for the next pair return before these loads do; they were requested during the last steps above.)
+    {
+      const int rgroup = wave % QH, sub = wave / QH;
+      const unsigned long long* mine = slots + 64 * rgroup + lane;
+      float m = kNegInf, acc = 0.f;
+      bool nan = false, ok = true;
+      int polls = 0;
+      for (int s0 = sub; s0 < S; s0 += kMergeWaves * kBatch) {
+        unsigned long long w[kBatch];
+        for (;;) {
+          bool all = true;
+#pragma unroll
+          for (int i = 0; i < kBatch; ++i) {
+            const int sidx = s0 + i * kMergeWaves;
+            w[i] = (sidx < S) ? __hip_atomic_load(mine + (int64_t)sidx * kRowsWg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                              : (((unsigned long long)round_no << 32) | 0xff800000u);   // -inf: adds nothing
+          }
+#pragma unroll
+          for (int i = 0; i < kBatch; ++i) all = all && ((unsigned)(w[i] >> 32) == round_no);
+          if (all || (FCR_FUSED_DBG & 3)) break;
+          if (++polls > spin_limit) {
+            ok = false;
+            break;
+          }
+          __builtin_amdgcn_s_sleep(8);
+        }
+        if (!ok) break;
+        float v[kBatch];
+#pragma unroll
+        for (int i = 0; i < kBatch; ++i) v[i] = __builtin_bit_cast(float, (unsigned)w[i]);
         float bm = v[0];
 #pragma unroll
-        for (int i = 1; i < 8; ++i) bm = fmaxf(bm, v[i]);
+        for (int i = 1; i < kBatch; ++i) bm = fmaxf(bm, v[i]);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) nan = nan || (v[i] != v[i]);
+        for (int i = 0; i < kBatch; ++i) nan = nan || (v[i] != v[i]);
         const float nm = fmaxf(m, bm);
         if (nm > kNegInf) {
-          acc *= fast_exp2(m - nm);
+          acc *= fast_exp2(m - nm);   // m = -inf: acc is 0 and stays 0
 #pragma unroll
-          for (int i = 0; i < 8; ++i) acc += fast_exp2(v[i] - nm);
+          for (int i = 0; i < kBatch; ++i) acc += fast_exp2(v[i] - nm);
           m = nm;
         }
       }
+      if (!ok) {
+        __hip_atomic_store(p.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        flag[1] = 0;
+      }
+      // a NaN partial (fmaxf drops it) makes the row's lse NaN
+      mrg[(sub * kRowsWg + 64 * rgroup + lane) * 2] = nan ? __builtin_nanf("") : m;
+      mrg[(sub * kRowsWg + 64 * rgroup + lane) * 2 + 1] = acc;
+    }
+    lds_barrier();
+    FCR_STAMP(3)
+    if (tid < kRowsWg) {
+      float m = kNegInf;
+      bool nan = false;
+#pragma unroll
+      for (int w = 0; w < kMergeWaves; ++w) {
+        const float mv = mrg[(w * kRowsWg + tid) * 2];
+        nan = nan || (mv != mv);
+        m = fmaxf(m, mv);
+      }
+      float acc = 0.f;
+#pragma unroll
+      for (int w = 0; w < kMergeWaves; ++w) {
+        const float mv = mrg[(w * kRowsWg + tid) * 2];
+        acc += (mv > kNegInf) ? mrg[(w * kRowsWg + tid) * 2 + 1] * fast_exp2(mv - m) : 0.f;
+      }
       const float lse = nan ? __builtin_nanf("") : ((m > kNegInf) ? m + fast_log2(acc) : kNegInf);
       rowv[tid] = -lse;
-      if (split == 0 && tid < p.M && met) p.lse[(int64_t)bh * p.M + tid] = lse;
+      if (split == 0 && tid < p.M) p.lse[(int64_t)bh * p.M + tid] = lse;   // (not meaningful if the team was not met)
     }
-    __syncthreads();
+    lds_barrier();
+    const bool met = flag[1] != 0;
+    if (tid == 0) flag[0] = 0;
+    if (!met) spin_limit = min(spin_limit, 64);   // the call has failed: later waits of this workgroup are short
+    // the queries of the next pair arrive while this one is finished from the registers
+    if (it + 1 < rounds) load_queries(bh + T, lane);
 
+    FCR_STAMP(4)
     // 4. probabilities, reduced down the rows
     f32x4 nl[4];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) nl[g] = *reinterpret_cast<const f32x4*>(rowv + 64 * half + 16 * g + qrow);
-    float* const osum = obuf + half * (kRes * kItemKeys);
+    for (int g = 0; g < 4; ++g) nl[g] = *reinterpret_cast<const f32x4*>(rowv + 64 * qh + 16 * g + qrow);
+    float* const osum = obuf + qh * (kRes * kItemKeys);
     float* const omax = osum + (MODE == kModeBoth ? kItemKeys : 0);
+    int c0b = c0;
+    asm volatile("" : "+s"(c0b));
 #pragma unroll
     for (int j = 0; j < KG; ++j) {
-      const int kbase = (c0 + j) * kChunk;
+      const int kbase = (c0b + j) * kChunk;
       const int key = kbase + 16 * wq + (lane & 15);
-      const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * half);
+      const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * qh);
       float vsum = 0.f, vmax = kNegInf;
       if (need_mask) {   // hidden entries stay hidden from a row whose lse is not a number
-        int first = CAUSAL ? key - p.c - 64 * half - qrow : -(1 << 30);
+        int first = CAUSAL ? key - p.c - 64 * qh - qrow : -(1 << 30);
         if (key >= p.N) first = 1 << 30;
 #pragma unroll
         for (int g = 0; g < 4; ++g)
@@ -1393,10 +1564,11 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
         if (lane < 16) omax[slot] = fast_exp2(vmax);
       }
     }
-    __syncthreads();
+    lds_barrier();
+    FCR_STAMP(5)
     void* const out_max = (MODE == kModeBoth) ? p.out2 : p.out;
     const float poison = __builtin_nanf("");
-    for (int i = tid; i < kItemKeys; i += kThreads * QH) {
+    for (int i = tid; i < kItemKeys; i += kNumThreads) {
       if (key0 + i < keys_end) {
         if (MODE != kModeMax) {
           float v = obuf[i];
@@ -1411,6 +1583,7 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
         }
       }
     }
+    FCR_STAMP(6)
     // the next writers of obuf, red, rowv and flag are behind the ring barriers of the next pair
   }
   ring_sync<0>();   // the loads past the last chunk write their zeros before the LDS is given back
@@ -1970,6 +2143,7 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   p.teams = 0;
   p.sync = nullptr;
   p.spin_limit = 0;
+  p.stagger = 0;
   return 0;
 }
 
@@ -1989,8 +2163,8 @@ int row_splits(int B, int H, int M, int N, int ksteps) {
 }
 
 // The single-sweep path (col_fused_kernel): 16-bit operands, rows of at most 256 bytes, at most 128 queries
-// and enough keys for the sweep to matter.  A (b,h) pair is shared by `splits` workgroups of kFusedChunks
-// chunks each; teams * splits workgroups are launched, never more than the chip holds at once.
+// and enough keys for the sweep to matter.  A (b,h) pair is shared by `splits` workgroups of 512 keys each;
+// teams * splits workgroups are launched, never more than the chip holds at once.
 constexpr int kFusedMinChunks = 16;   // 1024 keys
 struct FusedPlan {
   int qh;       // 1: 64 query rows per workgroup (256 threads, two per CU), 2: 128 (512 threads, one per CU)
@@ -2003,15 +2177,15 @@ bool fused_shape(int64_t bh, int M, int N, FusedPlan& f) {
   const int64_t nchunks = ((int64_t)N + kChunk - 1) / kChunk;
   if (M > 2 * 64 || nchunks < kFusedMinChunks) return false;
   f.qh = M > 64 ? 2 : 1;
-  const int cap = chip_cus() * (3 - f.qh);
-  const int64_t splits = (nchunks + kFusedChunks - 1) / kFusedChunks;
+  const int cap = chip_cus() * (3 - f.qh);   // two workgroups of 256 threads or one of 512 per CU
+  const int64_t splits = (nchunks + kFusedSteps - 1) / kFusedSteps;
   if (splits > cap) return false;
   f.splits = (int)splits;
   const int64_t teams = cap / splits;
   f.teams = (int)(teams < bh ? teams : bh);
   f.part_at = (bh * M + 63) / 64 * 64;
-  f.sync_at = f.part_at + 2ll * cap * 64 * f.qh;   // two sets of one slot of 64 * qh values per workgroup
-  f.floats = f.sync_at + ((int64_t)cap + 1) * 32;
+  f.sync_at = f.part_at + 2 * (2ll * cap * 64 * f.qh);   // two sets of one 64-bit slot per row and workgroup
+  f.floats = f.sync_at + 32;
   return true;
 }
 
@@ -2106,7 +2280,7 @@ void launch_col_fused_mode(const Params& p, bool causal, hipStream_t s) {
   else hipLaunchKernelGGL((col_fused_kernel<DT, KS, false, MODE, QH>), grid, block, 0, s, p);
 }
 
-// mode: kModeSum or kModeMax, + 4 for the eight-wave form (more than 64 queries)
+// mode: kModeSum or kModeMax, + 4 for more than 64 queries
 template <int DT, int KS>
 void launch_col_fused(const Params& p, bool causal, int mode, hipStream_t s) {
   const int m = mode & 3;
@@ -2431,9 +2605,10 @@ int whole_call(const void* q, const void* k, void* out, const ResultSpec& res, f
       p.inv_m = 1.0f / (float)M;
     }
     p.stream_once = ((int64_t)p.bh_count * N * p.dgran * 16 >= (1ll << 30)) ? 1 : 0;
-    const int words = (f.teams + 1) * 32;   // the teams' counters and the error word start at zero
+    const int words = (int)(f.floats - f.part_at);   // the slots and the error word start at zero
     fcr_detail::fused_refused = false;
-    launch_sweeps(dtype, 3, p, ksteps, causal != 0, mode | (f.qh == 2 ? 4 : 0), s, p.sync, words);
+    launch_sweeps(dtype, 3, p, ksteps, causal != 0, mode | (f.qh == 2 ? 4 : 0), s, reinterpret_cast<unsigned*>(p.part),
+                  words);
     if (!fcr_detail::fused_refused) return launched("col_fused_kernel");
   }
   rc = fcr_row_lse(q, k, ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream);
@@ -2545,8 +2720,8 @@ int fcr_colreduce_status(const float* lse_ws, int dtype, int B, int H, int M, in
   if (dtype == FCR_DTYPE_F32 || ksteps_of(dtype, D) > 4 || !fused_shape((int64_t)B * H, M, N, f)) return 0;
   unsigned word = 0;
   hipStream_t s = static_cast<hipStream_t>(stream);
-  hipError_t e = hipMemcpyAsync(&word, reinterpret_cast<const unsigned*>(lse_ws + f.sync_at) + 32 * f.teams,
-                                sizeof(word), hipMemcpyDeviceToHost, s);
+  hipError_t e = hipMemcpyAsync(&word, reinterpret_cast<const unsigned*>(lse_ws + f.sync_at), sizeof(word),
+                                hipMemcpyDeviceToHost, s);
   if (e == hipSuccess) e = hipStreamSynchronize(s);
   if (e != hipSuccess) {
     snprintf(g_err, sizeof(g_err), "reading the status word failed: %s", hipGetErrorString(e));

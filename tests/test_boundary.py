@@ -38,9 +38,9 @@ def test_version_and_sizes():
     assert lib.fcr_lse_bytes(2, 3, 5, 7, 64) == 2 * 3 * 5 * 4
     assert lib.fcr_lse_bytes(1, 32, 8192, 8192, 128) == 32 * 8192 * 4      # enough row tiles: no scratch
     assert lib.fcr_lse_bytes(1, 32, 512, 16384, 128) == 32 * 512 * 4 * 9   # 8 key ranges + the result
-    # few queries, many keys (256 CUs assumed without a device): the result, two sets of partial values
-    # for one workgroup per CU of 128 rows, a counter line per workgroup and the status line
-    assert lib.fcr_lse_bytes(1, 32, 128, 4096, 128) == (32 * 128 + 2 * 256 * 128 + 257 * 32) * 4
+    # few queries, many keys (256 CUs assumed without a device): the result, two sets of 64-bit slots for
+    # one workgroup per CU of 128 rows, and the status line
+    assert lib.fcr_lse_bytes(1, 32, 128, 4096, 128) == (32 * 128 + 2 * 2 * 256 * 128 + 32) * 4
     assert lib.fcr_lse_bytes(-1, 3, 5, 7, 8) == 0 and lib.fcr_lse_bytes(1, 3, 0, 7, 8) == 0
 
 
