@@ -34,6 +34,8 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <type_traits>
+
 #include "fcr.h"
 
 // The file can be compiled whole, or in parts that are linked together (the build script does that to
@@ -1102,7 +1104,7 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
 
 // ---------------------------------------------------------------------------------------------
 // Both sweeps in one for at most 128 query rows against many keys: the keys are read from memory ONCE.
-// A team of p.splits workgroups shares a (b,h) pair; workgroup s of the team owns kFusedSteps chunks of
+// A team of p.splits workgroups shares a (b,h) pair; workgroup s of the team owns 16 or 8 chunks of
 // 64 keys; wave w takes keys [16 (w & 3), +16) of each chunk against 64 queries (as in col_small_kernel).
 // Per pair ("item") a workgroup
 //   1. streams its keys through the LDS ring and computes their scores; the scaled scores STAY IN REGISTERS
@@ -1121,7 +1123,10 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
 // flight.  Traffic between workgroups uses device-scope atomics only (relaxed stores and loads, performed
 // where every workgroup of the device sees them); partial slots alternate between two sets by the parity
 // of the round: a workgroup can be at most one round ahead of the slowest of its team.
+// chunks of 64 keys per workgroup and pair
+__host__ __device__ constexpr int fused_chunks(int qh) { return qh == 1 ? 16 : 8; }
 constexpr int kFusedSteps = 8;
+constexpr int kFusedThreads = 512;
 #ifndef FCR_FUSED_DBG
 #define FCR_FUSED_DBG 0
 #endif
@@ -1157,28 +1162,32 @@ __global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ 
   if (i < n) w[i] = 0u;
 }
 
-// kFusedSteps chunks of 64 keys per workgroup and pair.  Up to 64 queries (QH = 1): four waves, two
-// workgroups per CU.  Up to 128 (QH = 2): eight waves, waves 4-7 hold queries 64-127, one workgroup per CU.
-// Waves 0-3 load.
+// Eight waves, one workgroup per CU, eight steps per workgroup and pair.  Up to 64 queries (QH = 1, KH = 2):
+// a step is two chunks of 64 keys, waves 0-3 take (and load) the first, waves 4-7 the second.  Up to 128
+// queries (QH = 2, KH = 1): a step is one chunk, waves 4-7 hold queries 64-127, waves 0-3 load.
 template <int DT, int KS, bool CAUSAL, int MODE, int QH>
-__global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Params p) {
+__global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Params p) {
   constexpr int KG = kFusedSteps;
-  constexpr int NS = 4 * QH;                     // ring stages (chunks): 66 KiB per workgroup, or 133
-  using Rg = Ring<KS, NS>;                       // waves 0-3 load, four loads of 1 KiB each per chunk for 256-byte rows
-  constexpr int kNumThreads = kThreads * QH;
+  constexpr int KH = 3 - QH;                     // chunks per step
+  constexpr int NS = (QH == 1) ? 8 : 6;          // ring stages (chunks): 130 KiB or 98 KiB for 256-byte rows
+  using Rg = Ring<KS, NS>;                       // four loads of 1 KiB per loading wave and chunk for 256-byte rows
+  constexpr int kQBytes = QH * Rg::kRows;        // the queries of a pair, staged like a chunk of keys per 64 rows
+  constexpr int kNumThreads = kFusedThreads;
   constexpr int kRowsWg = 64 * QH;               // query rows a workgroup holds
-  constexpr int kItemKeys = KG * kChunk;
+  constexpr int kItemKeys = KG * KH * kChunk;
   constexpr int kRes = (MODE == kModeBoth) ? 2 : 1;
   constexpr int kObufFloats = QH * kRes * kItemKeys;
-  constexpr int kRedFloats = kWaves * QH * 64;
-  constexpr int kMergeWaves = 4;                 // waves per row that share the merge of the team's partial values
-  constexpr int kBatch = 8;                      // slots a lane fetches together: one round trip for teams of up to 32
+  constexpr int kRedFloats = 8 * 64;
+  constexpr int kMergeWaves = 8 / QH;            // waves per row that share the merge of the team's partial values
+  constexpr int kBatch = 4 * QH;                 // slots a lane fetches together: one round trip for teams of up to 32
   constexpr int kMrgFloats = kMergeWaves * kRowsWg * 2;
-  constexpr int kAhead = NS - 1;                 // chunks in flight in front of the one being computed
-  constexpr int kInFlight = (NS - 2) * Rg::kPer; // loads a loader wave may have outstanding when a step starts
-  // one LDS object (see col_small_kernel): ring | finished columns | per-wave row partials | merge | per-row values | flags
-  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes + (kObufFloats + kRedFloats + kMrgFloats + kRowsWg + 4) * 4];
-  float* const obuf = reinterpret_cast<float*>(smem + Rg::kBytes);
+  constexpr int kAhead = NS / KH - 1;            // steps in flight in front of the one being computed
+  constexpr int kInFlight = (NS / KH - 2) * Rg::kPer;   // loads a loading wave may have outstanding when a step starts
+  // (one LDS object: see col_small_kernel)
+  // one LDS object: ring | queries | finished columns | per-wave row partials | merge | per-row values | flags
+  __shared__ __attribute__((aligned(1024))) char smem[Rg::kBytes + kQBytes + (kObufFloats + kRedFloats + kMrgFloats + kRowsWg + 4) * 4];
+  char* const qlds = smem + Rg::kBytes;
+  float* const obuf = reinterpret_cast<float*>(smem + Rg::kBytes + kQBytes);
   float* const red = obuf + kObufFloats;
   float* const mrg = red + kRedFloats;
   float* const rowv = mrg + kMrgFloats;
@@ -1187,11 +1196,12 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
   const int tid0 = threadIdx.x, lane0 = tid0 & 63;   // (the loop over the pairs has its own copies, see there)
   const int wave = __builtin_amdgcn_readfirstlane(tid0 >> 6);
   const int qh = (QH == 2) ? (wave >> 2) : 0;    // which 64 queries
+  const int kh = (KH == 2) ? (wave >> 2) : 0;    // which chunk of a step
   const int wq = wave & 3;                       // which 16 keys of the chunk
-  const bool loader = (QH == 1) || (wave < 4);
+  const bool loader = (KH == 2) || (wave < 4);
   const int S = p.splits, T = p.teams;
   const int team = (int)blockIdx.x / S, split = (int)blockIdx.x - team * S;
-  const int c0 = split * KG;                     // first chunk of this workgroup's keys
+  const int c0 = split * (KG * KH);              // first chunk of this workgroup's keys
   const int key0 = c0 * kChunk;
   const int keys_end = min(p.N, key0 + kItemKeys);
   const int rounds = (p.bh_count - team + T - 1) / T;
@@ -1205,8 +1215,8 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
   rg.init(p.k_sr, p.dgran, lane0, 0);   // (for the fragment offsets; the loads are issued below)
   const bool once = p.stream_once != 0;
   auto stage_of = [&](int c) { return smem + ((uint32_t)c % NS) * Rg::kStage; };   // NS is a power of two
-  // The loaders walk the workgroup's stream of chunks with a running address: KG chunks of one pair, then
-  // the same range of keys of the next pair of the team.  Chunk number c goes to stage c % NS.
+  // The loaders walk the workgroup's stream of chunks with a running address: KG * KH chunks of one pair,
+  // then the same range of keys of the next pair of the team.  Chunk number c goes to stage c % NS.
   const int64_t chunk_bytes = (int64_t)kChunk * p.k_sr;
   const char* run_ptr = nullptr;
   int run_rows = 0, run_chunk = 0;
@@ -1231,12 +1241,16 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
     src_off[e] = (uint32_t)row * (uint32_t)p.k_sr + (uint32_t)c * 16u;
   }
   const uint32_t pat_bytes = (uint32_t)(kPat * Rg::kRowsPerLoad) * (uint32_t)p.k_sr;
-  auto issue_step = [&]() {
+  auto issue_step = [&]() {   // the wave's chunk of the next step
+    char* stage = stage_of(run_chunk + kh);
+    const char* src = run_ptr + (KH == 2 && kh ? chunk_bytes : 0);
+    const int live = rows_in_chunk(run_rows - kh * kChunk);
+    run_chunk += KH;        // (every wave keeps the cursor, only the loading ones issue)
+    run_ptr += KH * chunk_bytes;
+    run_rows -= KH * kChunk;
     if (!loader) return;
-    char* stage = stage_of(run_chunk);
-    const int live = rows_in_chunk(run_rows);
     const __amdgpu_buffer_rsrc_t view = __builtin_amdgcn_make_buffer_rsrc(
-        const_cast<char*>(run_ptr), 0, (int)((uint32_t)live * (uint32_t)p.k_sr), 0x00020000);
+        const_cast<char*>(src), 0, (int)((uint32_t)live * (uint32_t)p.k_sr), 0x00020000);
     uint32_t so[kPat];   // opaque copies: the kPer offsets are made per call, not kept in registers between calls
 #pragma unroll
     for (int e = 0; e < kPat; ++e) {
@@ -1256,54 +1270,78 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
         dma16<0>(view, off, stage + (lw * Rg::kPer + i) * 1024);
       }
     }
-    run_ptr += chunk_bytes;
-    run_rows -= kChunk;
-    ++run_chunk;
   };
-  run_to_pair(team);
-#pragma unroll
-  for (int i = 0; i < kAhead; ++i) issue_step();
+  int cons_chunk = 0;       // number of the next chunk to be computed (its stage: cons_chunk % NS)
 
   int qrows[4];
 #pragma unroll
   for (int g = 0; g < 4; ++g) qrows[g] = 64 * qh + 16 * g;
   u32x4 qf[4][KS];
-  // (like load_resident, but the zero padding of D comes from offsets outside the view instead of a select
-  // on the loaded value: nothing here waits for the data, which is first touched by the next pair's MFMAs)
-  auto load_queries = [&](int bh, int lane) {
+  // The queries of a pair go from memory to LDS like a chunk of keys (64 rows per stage-like tile, same
+  // swizzle), long before they are needed, and from there into the registers when the pair's sweep starts:
+  // no wave ever waits for them, and they take no registers between two sweeps.  Waves 0-3 load.
+  auto stage_queries = [&](int bh) {
+    if (wave >= 4) return;
     const int b = bh / p.H, h = bh - b * p.H;
     const char* qb = p.q + (int64_t)b * p.q_sb + (int64_t)h * p.q_sh;
-    const uint32_t roff = (uint32_t)(lane & 15) * (uint32_t)p.q_sr;
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const __amdgpu_buffer_rsrc_t view = rows_view(qb, p.q_sr, qrows[g], p.M);
+    for (int t = 0; t < QH; ++t) {
+      const int live = rows_in_chunk(p.M - 64 * t);
+      const __amdgpu_buffer_rsrc_t view = __builtin_amdgcn_make_buffer_rsrc(
+          const_cast<char*>(qb + (int64_t)(64 * t) * p.q_sr), 0, (int)((uint32_t)live * (uint32_t)p.q_sr), 0x00020000);
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int gi = ks * 4 + (lane >> 4);
-        qf[g][ks] = view_load16(view, gi < p.dgran ? roff + (uint32_t)gi * 16u : kPastEnd);
+      for (int i = 0; i < Rg::kPer; ++i) {
+        const int byte = (lw * Rg::kPer + i) * 1024 + lane0 * 16;
+        const int row = byte / Rg::kPitch;
+        const int c = ((byte % Rg::kPitch) / 16) ^ Rg::swz(row);
+        const uint32_t off = (c < p.dgran) ? (uint32_t)row * (uint32_t)p.q_sr + (uint32_t)c * 16u : kPastEnd;
+        dma16<0>(view, off, qlds + t * Rg::kRows + (lw * Rg::kPer + i) * 1024);
       }
     }
   };
-  load_queries(team, lane0);
+  auto read_queries = [&]() {
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) qf[g][ks] = rg.frag(qlds + qh * Rg::kRows, g >> 1, g & 1, ks);
+  };
+  // the first pair's queries, then the first steps of its keys: the loads return in this order, so the
+  // wait in front of the first step covers the queries
+  stage_queries(team);
+  run_to_pair(team);
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i) issue_step();
 
   // Register (g, r) of a lane is query 64*qh + 16g + qrow + r against the lane's key.  It takes part iff
   // the query exists and may see the key: 16g + r in [first, mlim).
   const int mlim0 = p.M - 64 * qh - qrow0;
   const bool ragged_rows = p.M < 64 * (qh + 1);
-  constexpr int kRowWaves = kWaves;   // row tid (tid < kRowsWg) is held by four waves: 0-3, or 4-7 for the rows from 64 on
+  constexpr int kRowWaves = 8 / QH;   // row tid (tid < kRowsWg) is held by all eight waves, or by 0-3 / 4-7 for rows below / from 64
 
 #if FCR_FUSED_DBG & 16
   long long* const stamps = reinterpret_cast<long long*>(p.out2);
 #define FCR_STAMP(n) if (stamps != nullptr && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 301) && it < 16) stamps[((blockIdx.x ? 1 : 0) * 16 + it) * 8 + (n)] = (long long)wall_clock64();
+#define FCR_STAMP2(n) if (stamps != nullptr && tid == 0 && blockIdx.x == 0 && it < 8) stamps[256 + it * 32 + (n)] = (long long)wall_clock64();
 #else
 #define FCR_STAMP(n)
+#define FCR_STAMP2(n)
 #endif
   for (int it = 0; it < rounds; ++it) {
     const int bh = team + it * T;
+    // What the registers keep per score: for column sums 2^score (step 4 is then one multiply-add per score),
+    // otherwise, or when a row's sum of 2^score is unusable, the score itself.  In the second case of a sum
+    // the scores are gone by the time it shows, and the keys of the pair are streamed once more.
     f32x4 sc[KG][4];
     f32x4 rs[4];   // per row (register) and key (lane): sum of 2^score over the steps
+    float my_lse = kNegInf;   // of row tid over this workgroup's keys, for tid < kRowsWg
+    // Steps 1 and the first half of 2, in two forms (KEEP: the registers end up holding the scores).  Returns
+    // whether some row's sum of 2^score is unusable.
+    auto sweep = [&](auto keep_tag) -> bool {
+    constexpr bool KEEP = decltype(keep_tag)::value;
+    if (KEEP) {
 #pragma unroll
-    for (int g = 0; g < 4; ++g) rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int g = 0; g < 4; ++g) rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    }
     {
     const int tid = tid0, lane = lane0, qrow = qrow0, mlim = mlim0;
     FCR_STAMP(0)
@@ -1314,10 +1352,15 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
     asm volatile("" : "+s"(c0a));
 #pragma unroll
     for (int j = 0; j < KG; ++j) {
+      FCR_STAMP2(3 * j)
       ring_sync<kInFlight>();   // the chunks of this step are visible, the stages of the step before are free
-      if (j + kAhead == KG) run_to_pair(bh + T);   // the chunks from here on belong to the next pair
+      FCR_STAMP2(3 * j + 1)
+      if (j + kAhead == KG) run_to_pair(bh + T);   // the steps from here on belong to the next pair
       issue_step();
-      const char* lds = stage_of(it * KG + j);
+      if (j == 0) read_queries();   // (staged at least a whole sweep ago; the barrier above has published them)
+      if (j == 1 && it + 1 < rounds) stage_queries(bh + T);   // every wave has read this pair's by now
+      FCR_STAMP2(3 * j + 2)
+      const char* lds = stage_of(cons_chunk + j * KH + kh);
 #pragma unroll
       for (int g = 0; g < 4; ++g) sc[j][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -1326,7 +1369,7 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
 #pragma unroll
         for (int g = 0; g < 4; ++g) sc[j][g] = mma<DT>(qf[g][ks], kfrag, sc[j][g]);
       }
-      const int kbase = (c0a + j) * kChunk;
+      const int kbase = (c0a + j * KH + kh) * kChunk;
       const int key = kbase + 16 * wq + (lane & 15);
       const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * qh);
       if (need_mask) {
@@ -1343,21 +1386,37 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
 #pragma unroll
         for (int g = 0; g < 4; ++g) sc[j][g] *= p.scale2;
       }
+      if (KEEP) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < 4; ++g)
 #pragma unroll
-        for (int r = 0; r < 4; ++r) rs[g][r] += fast_exp2(sc[j][g][r]);
+          for (int r = 0; r < 4; ++r) rs[g][r] += fast_exp2(sc[j][g][r]);
+      } else {   // (the row sums are taken after the loop: sixteen registers less while the queries are held)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sc[j][g][r] = (FCR_FUSED_DBG & 64) ? sc[j][g][r] + 1.0f : fast_exp2(sc[j][g][r]);
+      }
     }
+    cons_chunk += KG * KH;
     FCR_STAMP(1)
     }
-    // From here to the end of the pair, everything that depends on the thread is derived afresh from an
-    // opaque copy of its number: values kept for these steps across step 1 would take registers from the
-    // scores (and come back from scratch memory, a round trip each).
+    if (FCR_FUSED_DBG & 256) return false;
+    if (!KEEP) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        rs[g] = sc[0][g];
+#pragma unroll
+        for (int j = 1; j < KG; ++j) rs[g] += sc[j][g];
+      }
+    }
+    // From here on, everything that depends on the thread is derived afresh from an opaque copy of its
+    // number: values kept for these steps across step 1 would take registers from the scores (and come
+    // back from scratch memory, a round trip each).
     int tid_again = threadIdx.x;
     asm volatile("" : "+v"(tid_again));
     const int tid = tid_again, lane = tid & 63, qrow = 4 * (lane >> 4);
-    const int mlim = p.M - 64 * qh - qrow;
-    const float* const red_row = red + (tid >> 6) * (kWaves * 64) + (tid & 63);
+    const float* const red_row = red + (QH == 2 ? (tid >> 6) * (kWaves * 64) : 0) + (tid & 63);
 
     // 2. log-sum-exp of every row over this workgroup's keys.  The sums of 2^x were taken as the scores
     // came; they are good unless a sum left fp32's comfortable range (or a row saw no key at all), and then
@@ -1369,18 +1428,51 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
       if ((lane & 15) == 0) *reinterpret_cast<f32x4*>(red + wave * 64 + 16 * g + qrow) = rs[g];
     }
     lds_barrier();
-    float my_lse = kNegInf;   // of row tid over this workgroup's keys, for tid < kRowsWg
     if (tid < kRowsWg) {
       float l = 0.f;
 #pragma unroll
       for (int w = 0; w < kRowWaves; ++w) l += red_row[64 * w];
       my_lse = fast_log2(l);
-      const bool good = (l >= 8.6736174e-19f) && (l < kPosInf);   // 2^-60: flushed terms are far below the sum's last bit
+      // 2^-60 <= l < 2^100: terms flushed to zero are far below the sum's last bit, and 2^score times 2^-lse
+      // (the lse of all keys is at least this one) neither overflows nor loses anything above 2^-26
+      const bool good = (l >= 8.6736174e-19f) && (l < 1.2676506e30f);
       if (!good && tid < p.M) flag[0] = 1;   // (written by whoever finds a bad row; thread 0 resets it below)
       if (tid == 0) flag[1] = 1;
     }
     lds_barrier();
-    if (flag[0] != 0) {   // uniform over the workgroup
+    return flag[0] != 0;   // uniform over the workgroup
+    };   // sweep
+    bool keep_scores = (MODE != kModeSum);
+    bool bad_sum;
+    if (FCR_FUSED_DBG & 128) {   // the sweep alone
+      sweep(std::false_type());
+      if (sc[0][0][0] + sc[7][3][3] + rs[0][0] == 12345.f) p.lse[0] = 1.f;
+      continue;
+    }
+    if (MODE == kModeSum) {
+      bad_sum = sweep(std::false_type());
+      if (bad_sum) {
+        // once more through the keys of this pair: the loads in flight (for the next pair) land and are
+        // dropped, the loader goes back to this pair's first chunk and the ring starts afresh
+        ring_sync<0>();
+        if (tid0 == 0) flag[0] = 0;
+        stage_queries(bh);   // (the sweep above has already replaced them by the next pair's)
+        run_to_pair(bh);
+        cons_chunk = run_chunk;
+#pragma unroll
+        for (int i = 0; i < kAhead; ++i) issue_step();
+        keep_scores = true;
+        bad_sum = sweep(std::true_type());
+      }
+    } else {
+      bad_sum = sweep(std::true_type());
+    }
+    int tid_once_more = threadIdx.x;
+    asm volatile("" : "+v"(tid_once_more));
+    const int tid = tid_once_more, lane = tid & 63, qrow = 4 * (lane >> 4);
+    const int mlim = p.M - 64 * qh - qrow;
+    const float* const red_row = red + (QH == 2 ? (tid >> 6) * (kWaves * 64) : 0) + (tid & 63);
+    if (bad_sum) {
       f32x4 rm[4];
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -1489,30 +1581,33 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
     lds_barrier();
     FCR_STAMP(3)
     if (tid < kRowsWg) {
+      float mv[kMergeWaves], av[kMergeWaves];
+#pragma unroll
+      for (int w = 0; w < kMergeWaves; ++w) {
+        const float2 ma = *reinterpret_cast<const float2*>(mrg + (w * kRowsWg + tid) * 2);
+        mv[w] = ma.x;
+        av[w] = ma.y;
+      }
       float m = kNegInf;
       bool nan = false;
 #pragma unroll
       for (int w = 0; w < kMergeWaves; ++w) {
-        const float mv = mrg[(w * kRowsWg + tid) * 2];
-        nan = nan || (mv != mv);
-        m = fmaxf(m, mv);
+        nan = nan || (mv[w] != mv[w]);
+        m = fmaxf(m, mv[w]);
       }
+      const float ref = (m > kNegInf) ? m : 0.f;   // 2^(-inf - ref) = 0 times a finite sum: no branches
       float acc = 0.f;
 #pragma unroll
-      for (int w = 0; w < kMergeWaves; ++w) {
-        const float mv = mrg[(w * kRowsWg + tid) * 2];
-        acc += (mv > kNegInf) ? mrg[(w * kRowsWg + tid) * 2 + 1] * fast_exp2(mv - m) : 0.f;
-      }
+      for (int w = 0; w < kMergeWaves; ++w) acc = fmaf(av[w], fast_exp2(mv[w] - ref), acc);
       const float lse = nan ? __builtin_nanf("") : ((m > kNegInf) ? m + fast_log2(acc) : kNegInf);
-      rowv[tid] = -lse;
+      // what step 4 adds to a score, or multiplies 2^score by (nothing for rows that do not exist)
+      rowv[tid] = keep_scores ? -lse : ((tid < p.M && lse > kNegInf) ? fast_exp2(-lse) : 0.f);
       if (split == 0 && tid < p.M) p.lse[(int64_t)bh * p.M + tid] = lse;   // (not meaningful if the team was not met)
     }
     lds_barrier();
     const bool met = flag[1] != 0;
     if (tid == 0) flag[0] = 0;
     if (!met) spin_limit = min(spin_limit, 64);   // the call has failed: later waits of this workgroup are short
-    // the queries of the next pair arrive while this one is finished from the registers
-    if (it + 1 < rounds) load_queries(bh + T, lane);
 
     FCR_STAMP(4)
     // 4. probabilities, reduced down the rows
@@ -1523,13 +1618,32 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
     float* const omax = osum + (MODE == kModeBoth ? kItemKeys : 0);
     int c0b = c0;
     asm volatile("" : "+s"(c0b));
+    float vs[KG], vm[KG];   // per step: the lane's key, reduced over the lane's sixteen queries
 #pragma unroll
     for (int j = 0; j < KG; ++j) {
-      const int kbase = (c0b + j) * kChunk;
+      const int kbase = (c0b + j * KH + kh) * kChunk;
       const int key = kbase + 16 * wq + (lane & 15);
       const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * qh);
-      float vsum = 0.f, vmax = kNegInf;
-      if (need_mask) {   // hidden entries stay hidden from a row whose lse is not a number
+      f32x4 part = {0.f, 0.f, 0.f, 0.f};   // four independent chains
+      float vmax = kNegInf;
+      if (MODE == kModeSum && !keep_scores) {   // the registers hold 2^score, nl holds 2^-lse
+        if (need_mask) {
+          int first = CAUSAL ? key - p.c - 64 * qh - qrow : -(1 << 30);
+          if (key >= p.N) first = 1 << 30;
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const int o = 16 * g + r;
+              part[r] += (o >= first && o < mlim) ? sc[j][g][r] * nl[g][r] : 0.f;
+            }
+        } else {
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) if (!(FCR_FUSED_DBG & 32) || (g == 0 && r == 0)) part[r] = fmaf(sc[j][g][r], nl[g][r], part[r]);
+        }
+      } else if (need_mask) {   // hidden entries stay hidden from a row whose lse is not a number
         int first = CAUSAL ? key - p.c - 64 * qh - qrow : -(1 << 30);
         if (key >= p.N) first = 1 << 30;
 #pragma unroll
@@ -1539,7 +1653,7 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
             const int o = 16 * g + r;
             const float x = (o >= first && o < mlim) ? sc[j][g][r] + nl[g][r] : kNegInf;
             if (MODE != kModeSum) vmax = fmaxf(vmax, x);
-            if (MODE != kModeMax) vsum += fast_exp2(x);
+            if (MODE != kModeMax) part[r] += fast_exp2(x);
           }
       } else {
 #pragma unroll
@@ -1548,20 +1662,37 @@ __global__ __launch_bounds__(kThreads * QH, 2) void col_fused_kernel(const Param
           for (int r = 0; r < 4; ++r) {
             const float x = sc[j][g][r] + nl[g][r];
             if (MODE != kModeSum) vmax = fmaxf(vmax, x);
-            if (MODE != kModeMax) vsum += fast_exp2(x);
+            if (MODE != kModeMax) part[r] += fast_exp2(x);
           }
       }
-      // the four lane groups hold different queries of the same key
-      const int slot = j * kChunk + 16 * wq + lane;
-      if (MODE != kModeMax) {
-        vsum += __shfl_xor(vsum, 16);
-        vsum += __shfl_xor(vsum, 32);
-        if (lane < 16) osum[slot] = vsum;
+      vs[j] = (part[0] + part[1]) + (part[2] + part[3]);
+      vm[j] = vmax;
+    }
+    // the four lane groups hold different queries of the same key: two exchanges, all steps at once
+    if (MODE != kModeMax) {
+      float o[KG];
+#pragma unroll
+      for (int j = 0; j < KG; ++j) o[j] = __shfl_xor(vs[j], 16);
+#pragma unroll
+      for (int j = 0; j < KG; ++j) vs[j] += o[j];
+#pragma unroll
+      for (int j = 0; j < KG; ++j) o[j] = __shfl_xor(vs[j], 32);
+      if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < KG; ++j) osum[(j * KH + kh) * kChunk + 16 * wq + lane] = vs[j] + o[j];
       }
-      if (MODE != kModeSum) {
-        vmax = fmaxf(vmax, __shfl_xor(vmax, 16));
-        vmax = fmaxf(vmax, __shfl_xor(vmax, 32));
-        if (lane < 16) omax[slot] = fast_exp2(vmax);
+    }
+    if (MODE != kModeSum) {
+      float o[KG];
+#pragma unroll
+      for (int j = 0; j < KG; ++j) o[j] = __shfl_xor(vm[j], 16);
+#pragma unroll
+      for (int j = 0; j < KG; ++j) vm[j] = fmaxf(vm[j], o[j]);
+#pragma unroll
+      for (int j = 0; j < KG; ++j) o[j] = __shfl_xor(vm[j], 32);
+      if (lane < 16) {
+#pragma unroll
+        for (int j = 0; j < KG; ++j) omax[(j * KH + kh) * kChunk + 16 * wq + lane] = fast_exp2(fmaxf(vm[j], o[j]));
       }
     }
     lds_barrier();
@@ -2167,7 +2298,7 @@ int row_splits(int B, int H, int M, int N, int ksteps) {
 // teams * splits workgroups are launched, never more than the chip holds at once.
 constexpr int kFusedMinChunks = 16;   // 1024 keys
 struct FusedPlan {
-  int qh;       // 1: 64 query rows per workgroup (256 threads, two per CU), 2: 128 (512 threads, one per CU)
+  int qh;       // 1: 64 query rows per workgroup and 1024 keys per pair, 2: 128 rows and 512 keys
   int splits, teams;
   int64_t part_at, sync_at;   // where the partial row values and the counters start in the workspace, in floats
   int64_t floats;             // workspace size
@@ -2177,8 +2308,8 @@ bool fused_shape(int64_t bh, int M, int N, FusedPlan& f) {
   const int64_t nchunks = ((int64_t)N + kChunk - 1) / kChunk;
   if (M > 2 * 64 || nchunks < kFusedMinChunks) return false;
   f.qh = M > 64 ? 2 : 1;
-  const int cap = chip_cus() * (3 - f.qh);   // two workgroups of 256 threads or one of 512 per CU
-  const int64_t splits = (nchunks + kFusedSteps - 1) / kFusedSteps;
+  const int cap = chip_cus();   // one workgroup per CU
+  const int64_t splits = (nchunks + fused_chunks(f.qh) - 1) / fused_chunks(f.qh);
   if (splits > cap) return false;
   f.splits = (int)splits;
   const int64_t teams = cap / splits;
@@ -2264,12 +2395,12 @@ bool fits_per_cu(K kernel, int threads, int want) {
 
 template <int DT, int KS, int MODE, int QH>
 void launch_col_fused_mode(const Params& p, bool causal, hipStream_t s) {
-  const dim3 grid(p.total), block(kThreads * QH);
+  const dim3 grid(p.total), block(kFusedThreads);
   static int fits[2] = {-1, -1};   // asked once per kernel (the answer depends on its registers and LDS, not on the device of a kind)
   int f = __atomic_load_n(&fits[causal], __ATOMIC_RELAXED);
   if (f < 0) {
-    f = causal ? fits_per_cu(col_fused_kernel<DT, KS, true, MODE, QH>, kThreads * QH, 3 - QH)
-               : fits_per_cu(col_fused_kernel<DT, KS, false, MODE, QH>, kThreads * QH, 3 - QH);
+    f = causal ? fits_per_cu(col_fused_kernel<DT, KS, true, MODE, QH>, kFusedThreads, 1)
+               : fits_per_cu(col_fused_kernel<DT, KS, false, MODE, QH>, kFusedThreads, 1);
     __atomic_store_n(&fits[causal], f, __ATOMIC_RELAXED);
   }
   if (!f) {
