@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(_HERE, "libfcr.so")
 DTYPE_F16, DTYPE_BF16, DTYPE_F32 = 0, 1, 2
 REDUCE_SUM, REDUCE_MAX, REDUCE_MEAN = 0, 1, 2
 OPT_SINGLE_SWEEP, OPT_WAIT_POLLS = 0, 1
+E_WAIT = -8
 
 _I64x4 = ctypes.c_int64 * 4
 _lib = None

@@ -74,7 +74,6 @@ struct Params {
   int teams;
   unsigned* sync;    // error word; zero at launch, like the slots at `part`
   int spin_limit;    // polls of the counter after which a wait gives up
-  int stagger;       // > 0: every other team starts this many sleeps late (see col_fused_kernel)
 };
 // which: 0 = row statistics, 1 = column sweep, 2 = column sweep for few queries, 3 = both sweeps in one for few
 // queries, mode + 4 for more than 64 of them (2 and 3: 16-bit types only)
@@ -1104,32 +1103,39 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
 
 // ---------------------------------------------------------------------------------------------
 // Both sweeps in one for at most 128 query rows against many keys: the keys are read from memory ONCE.
-// A team of p.splits workgroups shares a (b,h) pair; workgroup s of the team owns 16 or 8 chunks of
-// 64 keys; wave w takes keys [16 (w & 3), +16) of each chunk against 64 queries (as in col_small_kernel).
-// Per pair ("item") a workgroup
-//   1. streams its keys through the LDS ring and computes their scores; the scaled scores STAY IN REGISTERS
-//      (16 per lane and step), and the sums of 2^score per row are taken on the way;
-//   2. turns the sums into the log-sum-exp of every row over its own keys and publishes the 64 or 128 values
-//      (sums that left fp32's comfortable range are redone from the registers the exact way, maximum first);
-//   3. meets the other workgroups of its team on an arrival counter in memory, reads their partial values
-//      and merges them into the rows' lse (every workgroup of the team does this merge for itself);
-//   4. turns its scores into probabilities, reduces them down the rows and stores its columns.
-// The grid is teams * splits workgroups and never more than the chip holds at once, so every workgroup of a
-// team is running when its partners wait for it; team t takes pairs t, t + teams, t + 2 teams, ..  The keys of the next pair
-// stream into the ring while a workgroup does steps 2-4.  A wait is bounded: after p.spin_limit polls the
-// workgroup gives up, sets the error word, stores NaN columns for that pair and goes on, so every
-// workgroup reaches its end whatever happens to the others.
-// The barriers between the steps wait for LDS only, so the keys in flight for the next pair stay in
-// flight.  Traffic between workgroups uses device-scope atomics only (relaxed stores and loads, performed
-// where every workgroup of the device sees them); partial slots alternate between two sets by the parity
-// of the round: a workgroup can be at most one round ahead of the slowest of its team.
+// A team of p.splits workgroups shares a (b,h) pair; workgroup s of the team owns 16 chunks of 64 keys (8
+// with more than 64 queries); a wave takes 16 keys of a chunk against 64 queries (as in col_small_kernel).
+// Per pair a workgroup
+//   1. streams its keys through the LDS ring and computes their scores, which STAY IN REGISTERS (16 per
+//      lane and step): for column sums as 2^score, otherwise (maxima) as the scaled scores themselves;
+//   2. sums 2^score per row, turns the sums into the log-sum-exp of every row over its own keys and
+//      publishes the 64 or 128 values.  A sum outside [2^-60, 2^100) (scores far from zero, a row that
+//      sees none of these keys, a NaN) is not trusted: the scores are then reduced the exact way, row
+//      maximum first -- from the registers if they hold scores, else after a second sweep over the same
+//      keys that keeps the scores;
+//   3. reads the values the other workgroups of its team have published for this pair and merges them
+//      into the rows' lse (every workgroup of the team does this merge for itself);
+//   4. turns what it kept into probabilities (2^score * 2^-lse: one multiply-add per score), reduces them
+//      down the rows and stores its columns.
+// The grid is teams * splits workgroups and never more than one per CU, so every workgroup of a team is
+// running when its partners wait for it; team t takes pairs t, t + teams, t + 2 teams, ..  The first keys
+// of the next pair stream into the ring while a workgroup does steps 2-4, and the next pair's queries are
+// staged in LDS a whole sweep ahead.  A wait is bounded: after p.spin_limit polls the workgroup gives up,
+// sets the error word, stores NaN columns for that pair and goes on, so every workgroup reaches its end
+// whatever happens to the others.
+// Between workgroups: a partial value travels together with the number of its round as ONE 64-bit word,
+// written and read with device-scope relaxed atomics (performed where every workgroup of the device
+// sees them), so a word that shows the round shows the value; there is no counter, no fence and nobody
+// waits for a store to complete.  The slots start at zero (a small kernel in front clears them), rounds
+// count from 1, and the slots alternate between two sets by the parity of the round: a workgroup can be at
+// most one round ahead of the slowest of its team.  The barriers between the steps wait for LDS only, so
+// the keys in flight stay in flight.
+// Registers are the limit (128 for the scores, 64 for the queries during step 1): what depends on the
+// thread is derived again after step 1 from opaque copies instead of being kept across it.
 // chunks of 64 keys per workgroup and pair
 __host__ __device__ constexpr int fused_chunks(int qh) { return qh == 1 ? 16 : 8; }
 constexpr int kFusedSteps = 8;
 constexpr int kFusedThreads = 512;
-#ifndef FCR_FUSED_DBG
-#define FCR_FUSED_DBG 0
-#endif
 
 template <int CTRL>
 __device__ __forceinline__ float dpp_row(float v) {
@@ -1318,14 +1324,6 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
   const bool ragged_rows = p.M < 64 * (qh + 1);
   constexpr int kRowWaves = 8 / QH;   // row tid (tid < kRowsWg) is held by all eight waves, or by 0-3 / 4-7 for rows below / from 64
 
-#if FCR_FUSED_DBG & 16
-  long long* const stamps = reinterpret_cast<long long*>(p.out2);
-#define FCR_STAMP(n) if (stamps != nullptr && tid == 0 && (blockIdx.x == 0 || blockIdx.x == 301) && it < 16) stamps[((blockIdx.x ? 1 : 0) * 16 + it) * 8 + (n)] = (long long)wall_clock64();
-#define FCR_STAMP2(n) if (stamps != nullptr && tid == 0 && blockIdx.x == 0 && it < 8) stamps[256 + it * 32 + (n)] = (long long)wall_clock64();
-#else
-#define FCR_STAMP(n)
-#define FCR_STAMP2(n)
-#endif
   for (int it = 0; it < rounds; ++it) {
     const int bh = team + it * T;
     // What the registers keep per score: for column sums 2^score (step 4 is then one multiply-add per score),
@@ -1344,7 +1342,6 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     }
     {
     const int tid = tid0, lane = lane0, qrow = qrow0, mlim = mlim0;
-    FCR_STAMP(0)
     // 1. scores of this workgroup's keys, scaled, hidden ones at -inf
     // (what the mask needs is derived afresh from an opaque copy of c0 here and in step 4: kept across the
     // steps, or hoisted out of the loop over the pairs, it would cost registers that the scores need)
@@ -1352,14 +1349,11 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     asm volatile("" : "+s"(c0a));
 #pragma unroll
     for (int j = 0; j < KG; ++j) {
-      FCR_STAMP2(3 * j)
       ring_sync<kInFlight>();   // the chunks of this step are visible, the stages of the step before are free
-      FCR_STAMP2(3 * j + 1)
       if (j + kAhead == KG) run_to_pair(bh + T);   // the steps from here on belong to the next pair
       issue_step();
       if (j == 0) read_queries();   // (staged at least a whole sweep ago; the barrier above has published them)
       if (j == 1 && it + 1 < rounds) stage_queries(bh + T);   // every wave has read this pair's by now
-      FCR_STAMP2(3 * j + 2)
       const char* lds = stage_of(cons_chunk + j * KH + kh);
 #pragma unroll
       for (int g = 0; g < 4; ++g) sc[j][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -1395,13 +1389,11 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
 #pragma unroll
         for (int g = 0; g < 4; ++g)
 #pragma unroll
-          for (int r = 0; r < 4; ++r) sc[j][g][r] = (FCR_FUSED_DBG & 64) ? sc[j][g][r] + 1.0f : fast_exp2(sc[j][g][r]);
+          for (int r = 0; r < 4; ++r) sc[j][g][r] = fast_exp2(sc[j][g][r]);
       }
     }
     cons_chunk += KG * KH;
-    FCR_STAMP(1)
     }
-    if (FCR_FUSED_DBG & 256) return false;
     if (!KEEP) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
@@ -1444,11 +1436,6 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     };   // sweep
     bool keep_scores = (MODE != kModeSum);
     bool bad_sum;
-    if (FCR_FUSED_DBG & 128) {   // the sweep alone
-      sweep(std::false_type());
-      if (sc[0][0][0] + sc[7][3][3] + rs[0][0] == 12345.f) p.lse[0] = 1.f;
-      continue;
-    }
     if (MODE == kModeSum) {
       bad_sum = sweep(std::false_type());
       if (bad_sum) {
@@ -1524,7 +1511,6 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
       __hip_atomic_store(slots + (int64_t)split * kRowsWg + tid,
                          ((unsigned long long)round_no << 32) | __builtin_bit_cast(unsigned, my_lse), __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
-    FCR_STAMP(2)
     // All waves share the team's slots: lane = row, the waves of a row take every kMergeWaves-th slot, poll
     // until it carries this round, and fold the values into (max, sum).  (The keys a wave has in flight
     // for the next pair return before these loads do; they were requested during the last steps above.)
@@ -1546,7 +1532,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
           }
 #pragma unroll
           for (int i = 0; i < kBatch; ++i) all = all && ((unsigned)(w[i] >> 32) == round_no);
-          if (all || (FCR_FUSED_DBG & 3)) break;
+          if (all) break;
           if (++polls > spin_limit) {
             ok = false;
             break;
@@ -1579,7 +1565,6 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
       mrg[(sub * kRowsWg + 64 * rgroup + lane) * 2 + 1] = acc;
     }
     lds_barrier();
-    FCR_STAMP(3)
     if (tid < kRowsWg) {
       float mv[kMergeWaves], av[kMergeWaves];
 #pragma unroll
@@ -1601,15 +1586,14 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
       for (int w = 0; w < kMergeWaves; ++w) acc = fmaf(av[w], fast_exp2(mv[w] - ref), acc);
       const float lse = nan ? __builtin_nanf("") : ((m > kNegInf) ? m + fast_log2(acc) : kNegInf);
       // what step 4 adds to a score, or multiplies 2^score by (nothing for rows that do not exist)
-      rowv[tid] = keep_scores ? -lse : ((tid < p.M && lse > kNegInf) ? fast_exp2(-lse) : 0.f);
+      // (a NaN lse stays a NaN factor: the row's visible columns become NaN, as in the other kernels)
+      rowv[tid] = keep_scores ? -lse : ((tid < p.M && lse != kNegInf) ? fast_exp2(-lse) : 0.f);
       if (split == 0 && tid < p.M) p.lse[(int64_t)bh * p.M + tid] = lse;   // (not meaningful if the team was not met)
     }
     lds_barrier();
     const bool met = flag[1] != 0;
     if (tid == 0) flag[0] = 0;
     if (!met) spin_limit = min(spin_limit, 64);   // the call has failed: later waits of this workgroup are short
-
-    FCR_STAMP(4)
     // 4. probabilities, reduced down the rows
     f32x4 nl[4];
 #pragma unroll
@@ -1641,7 +1625,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
 #pragma unroll
           for (int g = 0; g < 4; ++g)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) if (!(FCR_FUSED_DBG & 32) || (g == 0 && r == 0)) part[r] = fmaf(sc[j][g][r], nl[g][r], part[r]);
+            for (int r = 0; r < 4; ++r) part[r] = fmaf(sc[j][g][r], nl[g][r], part[r]);
         }
       } else if (need_mask) {   // hidden entries stay hidden from a row whose lse is not a number
         int first = CAUSAL ? key - p.c - 64 * qh - qrow : -(1 << 30);
@@ -1696,7 +1680,6 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
       }
     }
     lds_barrier();
-    FCR_STAMP(5)
     void* const out_max = (MODE == kModeBoth) ? p.out2 : p.out;
     const float poison = __builtin_nanf("");
     for (int i = tid; i < kItemKeys; i += kNumThreads) {
@@ -1714,7 +1697,6 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
         }
       }
     }
-    FCR_STAMP(6)
     // the next writers of obuf, red, rowv and flag are behind the ring barriers of the next pair
   }
   ring_sync<0>();   // the loads past the last chunk write their zeros before the LDS is given back
@@ -2274,7 +2256,6 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
   p.teams = 0;
   p.sync = nullptr;
   p.spin_limit = 0;
-  p.stagger = 0;
   return 0;
 }
 

@@ -27,7 +27,8 @@ def test_library_exports_every_declared_symbol():
     names = _declared_symbols()
     assert {"fcr_version", "fcr_last_error", "fcr_lse_bytes", "fcr_row_lse", "fcr_col_reduce",
             "fcr_col_reduce_sum_max", "fcr_pack_f32", "fcr_colreduce", "fcr_colreduce_static",
-            "fcr_colreduce_to", "fcr_topk_mask", "fcr_topk_mask_ws", "fcr_topk_bytes"} <= set(names)
+            "fcr_colreduce_to", "fcr_topk_mask", "fcr_topk_mask_ws", "fcr_topk_bytes", "fcr_set_option",
+            "fcr_colreduce_status"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
 
@@ -90,6 +91,19 @@ def test_c_abi_rejects_bad_arguments_without_a_device(fn):
     with pytest.raises(_lib.FcrError) as e:
         _lib.check(_call(lib, fn, D=12))
     assert e.value.code == -3 and "multiple of 8" in str(e.value)
+
+
+def test_options_and_status_reject_bad_arguments_without_a_device():
+    lib = _lib.load()
+    assert lib.fcr_set_option(99, 1) == -3
+    assert lib.fcr_set_option(_lib.OPT_WAIT_POLLS, -5) == -3
+    assert lib.fcr_set_option(_lib.OPT_SINGLE_SWEEP, 1) == 0 and lib.fcr_set_option(_lib.OPT_WAIT_POLLS, 1 << 20) == 0
+    assert lib.fcr_colreduce_status(None, 0, 1, 1, 8, 8, 64, None) == -1
+    assert lib.fcr_colreduce_status(16, 0, 1, 1, 0, 8, 64, None) == -3
+    # problems that never take the single sweep have nothing to report: no device is asked
+    assert lib.fcr_colreduce_status(16, 0, 1, 1, 512, 512, 64, None) == 0      # more than 128 queries
+    assert lib.fcr_colreduce_status(16, 2, 1, 1, 64, 4096, 64, None) == 0      # fp32 operands
+    assert lib.fcr_colreduce_status(16, 0, 1, 1, 64, 512, 64, None) == 0       # fewer than 1024 keys
 
 
 def test_pack_f32_rejects_bad_arguments_without_a_device():

@@ -312,6 +312,165 @@ def test_key_operand_beyond_4_gib():
             torch.testing.assert_close(got.cpu(), want, rtol=2e-3, atol=0, msg=lambda m: f"{red} causal={causal}: {m}")
 
 
+# --- the single sweep for few queries against many keys (keys read once) -------------------------------------
+def _c_abi_colreduce(q, k, red, causal, scale=None):
+    """fcr_colreduce through ctypes on device tensors; returns (out [B,H,N] fp32, lse [B,H,M] fp32, status)."""
+    from flash_colreduce_amd import _lib
+    lib = _lib.load()
+    b, h, m, d = q.shape
+    n = k.shape[2]
+    out = torch.empty(b * h, n, device="cuda")
+    lse = torch.empty(lib.fcr_lse_bytes(b, h, m, n, d) // 4, device="cuda")
+    dt = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16}[q.dtype]
+    _lib.check(lib.fcr_colreduce(q.data_ptr(), k.data_ptr(), out.data_ptr(), lse.data_ptr(), dt, b, h, m, n, d,
+                                 _lib.strides4(q.stride()), _lib.strides4(k.stride()),
+                                 float(scale if scale is not None else 1 / math.sqrt(d)),
+                                 _lib.REDUCE_MAX if red == "max" else _lib.REDUCE_SUM, int(causal), None))
+    status = lib.fcr_colreduce_status(lse.data_ptr(), dt, b, h, m, n, d, None)
+    return out.view(b, h, n), lse[: b * h * m].view(b, h, m), status
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("b,h,m,n,d", [
+    (1, 2, 64, 1024, 128),     # the smallest problem that takes the single sweep: one workgroup per pair
+    (1, 3, 64, 16384, 128),    # teams of 16 workgroups
+    (2, 3, 128, 4096, 128),    # two query halves, teams of 8
+    (3, 5, 40, 3001, 64),      # ragged queries and keys, a partial last chunk
+    (1, 2, 100, 5000, 72),     # two halves, the second ragged; D not a multiple of 32
+    (2, 7, 17, 2100, 16),      # rows of 32 bytes
+    (1, 1, 1, 70000, 128),     # one query, 69 workgroups on one pair
+    (40, 16, 64, 2048, 32),    # 640 pairs for 128 teams: five rounds per workgroup
+])
+def test_single_sweep(b, h, m, n, d, causal, dtype):
+    """At most 128 queries against at least 1024 keys: one sweep over the keys computes the row statistics
+    and the columns (col_fused_kernel).  Sum, mean and max against the oracle through the operator; the
+    row statistics and the status word through the C ABI; and the two-kernel path on the same inputs."""
+    from flash_colreduce_amd import _lib
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=b + h + m + n, dtype=dtype)
+    qd, kd = q.cuda(), k.cuda()
+    what = f"single sweep b{b} h{h} m{m} n{n} d{d} {dtype}"
+    run_all(q, k, causal, what=what)
+    got, lse, status = _c_abi_colreduce(qd, kd, "sum", causal)
+    assert status == 0
+    torch.testing.assert_close(lse.double().cpu(), row_lse2_ref(q, k, causal), rtol=0, atol=3e-4)
+    lib = _lib.load()
+    lib.fcr_set_option(_lib.OPT_SINGLE_SWEEP, 0)
+    try:
+        two, lse2, _ = _c_abi_colreduce(qd, kd, "sum", causal)
+    finally:
+        lib.fcr_set_option(_lib.OPT_SINGLE_SWEEP, 1)
+    torch.testing.assert_close(got, two, rtol=2e-5, atol=1e-7)
+    torch.testing.assert_close(lse, lse2, rtol=0, atol=2e-5)
+    assert torch.equal(got, _c_abi_colreduce(qd, kd, "sum", causal)[0])   # no atomic adds: repeatable bit for bit
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m", [64, 128])
+def test_single_sweep_scores_far_from_zero(m, causal):
+    """Row sums of 2^score that overflow or vanish in fp32 (an enormous aligned key late in the sweep, rows
+    whose scores are all around -190, unscaled scores): the workgroup sweeps its keys a second time keeping
+    the scores and reduces them maximum first."""
+    b, h, n, d = 1, 3, 4096, 64
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=9)
+    q, k = q.float(), k.float()
+    k[:, 0, 3000] = 40.0 * q[:, 0, 50]
+    k[:, 0, 3001] = -40.0 * q[:, 0, 50]
+    k[:, 1] = -3.0 * q[:, 1, :1] + 0.1 * k[:, 1]
+    k[:, 1, 3500:] *= 0.0
+    for scale in (None, 1.0):
+        run_all(q.half(), k.half(), causal, scale=scale, what=f"single sweep, far scores, m{m} scale={scale}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_single_sweep_nan_and_inf_inputs(causal):
+    """As test_nan_and_inf_inputs, on a shape that takes the single sweep: NaN rows make the columns they
+    see NaN and leave the others alone; the maxima are compared where no NaN row looks."""
+    b, h, m, n, d = 1, 4, 100, 2600, 64
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=56)
+    q, k = q.clone(), k.clone()
+    q[0, 0, 70, 5] = float("nan")
+    q[0, 1, 20, 3] = float("inf")
+    k[0, 2, 1000, 7] = float("-inf")
+    c = max(n - m, 0)
+    scores = torch.einsum("bhmd,bhnd->bhmn", q.float(), k.float())
+    vis = (torch.arange(m)[:, None] + c >= torch.arange(n)[None, :]) if causal else torch.ones(m, n, dtype=torch.bool)
+    bad = ((torch.isnan(scores) | (scores == float("inf"))) & vis).any(-1)
+    assert bad[0, 0].sum() == 1 and bad[0, 1].sum() == 1 and bad[0, 2].sum() > 10 and not bad[0, 3].any()
+    nan_cols = (bad[..., None] & vis).any(-2)
+    q_clean = torch.where(bad[..., None], torch.zeros_like(q), q)
+    k_clean = torch.nan_to_num(k, neginf=0.0)
+    qd, kd = q.cuda(), k.cuda()
+    for red in REDUCTIONS:
+        got = fca.flash_colreduce(qd, kd, red, is_causal=causal, out_dtype=torch.float32).cpu()
+        want = colreduce_ref(q_clean, k_clean, red, causal)
+        if red != "max":
+            assert torch.equal(torch.isnan(got), nan_cols), red
+        ok = ~nan_cols
+        ok[0, 2] = False
+        if causal:
+            assert ok[0, 0].any() and ok[0, 1].any()
+        check(got[ok], want[ok], red, f"single sweep, columns no NaN row sees, causal={causal}")
+
+
+def test_single_sweep_bounded_wait():
+    """The wait for the team is bounded from the host: with a limit of zero polls a workgroup whose partners
+    have not all published gives up at once, stores NaN for its columns of that pair, sets the status word
+    and goes on; every workgroup ends normally.  What is not NaN is right, the status says whether anything
+    is, and the next call with the usual limit is clean."""
+    from flash_colreduce_amd import _lib
+    lib = _lib.load()
+    b, h, m, n, d = 4, 16, 64, 8192, 64
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=5)
+    qd, kd = q.cuda(), k.cuda()
+    want = colreduce_ref(q, k, "sum", True)
+    assert lib.fcr_set_option(_lib.OPT_WAIT_POLLS, 0) == 0
+    try:
+        got, _, status = _c_abi_colreduce(qd, kd, "sum", True)
+    finally:
+        assert lib.fcr_set_option(_lib.OPT_WAIT_POLLS, 1 << 20) == 0
+    got = got.cpu()
+    gave_up = torch.isnan(got)
+    assert status == (_lib.E_WAIT if gave_up.any() else 0), (status, int(gave_up.sum()))
+    if status:
+        assert b"gave up waiting" in lib.fcr_last_error()
+    torch.testing.assert_close(got[~gave_up], want[~gave_up], rtol=2e-3, atol=1e-5)
+    got, _, status = _c_abi_colreduce(qd, kd, "sum", True)
+    assert status == 0
+    check(got, want, "sum", "after the limit is restored")
+    assert lib.fcr_set_option(7, 1) == -3 and lib.fcr_set_option(_lib.OPT_WAIT_POLLS, -1) == -3
+
+
+def test_single_sweep_under_graph_capture():
+    """The single sweep (a small kernel that clears the slots, then the sweep) captured and replayed."""
+    b, h, m, n, d = 2, 8, 64, 4096, 128
+    qs = torch.zeros(b, h, m, d, device="cuda", dtype=torch.float16)
+    ks = torch.zeros(b, h, n, d, device="cuda", dtype=torch.float16)
+    q0, k0 = _inputs.randn_pair(b, h, m, n, d, seed=31)
+    qs.copy_(q0)
+    ks.copy_(k0)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fca.flash_colreduce(qs, ks, "mean", True, out_dtype=torch.float32)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fca.flash_colreduce(qs, ks, "mean", True, out_dtype=torch.float32)
+    for seed in (32, 33, 34):
+        q1, k1 = _inputs.randn_pair(b, h, m, n, d, seed=seed)
+        qs.copy_(q1)
+        ks.copy_(k1)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = out.clone()
+        eager = fca.flash_colreduce(qs, ks, "mean", True, out_dtype=torch.float32)
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), seed
+        check(got, colreduce_ref(q1, k1, "mean", True), "mean", f"single sweep, graph replay seed {seed}")
+
+
 @pytest.mark.parametrize("causal", [False, True])
 def test_explicit_and_negative_scale(causal):
     q, k = _inputs.randn_pair(1, 4, 200, 333, 64, seed=21)
