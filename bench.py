@@ -21,6 +21,10 @@ configs      the five named workloads of the benchmark set: ms per call (events,
              calls of the same workload), TFLOP/s by the
              metric's convention, fraction of the MFMA (and, for the decode-shaped one, HBM) roofline,
              the CPU oracle timed on a sample of heads, and the tolerance verdict per reduction.
+             `kernel_us` is the same problem through the C ABI with preallocated buffers, many calls back to
+             back between two events: the time of the call's kernels on the GPU as long as the host issues a
+             call faster than that (`host_issue_us`); `ms` is the Python operator, torch allocations included.
+             `--configs 2,3` restricts the set (and `--no-headline` skips the headline) for profiler runs.
 """
 from __future__ import annotations
 
@@ -37,7 +41,9 @@ PEAK_FP16_DENSE_TFLOPS = 2516.6  # 256 CU x 2.4 GHz x 4096 flop/CU/clk, MI355X p
 PEAK_HBM_TBPS = 8.0
 # HBM bytes per launch on the headline workload, from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs
 # scaled by the same counters on a 256 MiB device copy (FETCH unit 2 KiB, WRITE unit 1 KiB);
-# the summary of those runs is profiles/headline_causal_8192_fp16.md.
+# the summary of those runs is profiles/headline_causal_8192_fp16.md.  Against the 135.3 MB a launch has
+# to move (q, k, the fp32 result) that is 1.70 times the bytes for the row sweep and 1.48 for the column
+# sweep: streamed tiles that several workgroups ask for and that do not all meet in a cache.
 HBM_TRAFFIC_BYTES = {"row_lse_kernel": 229.5e6 + 1.05e6, "col_reduce_kernel": 199.7e6 + 1.05e6}
 CONDITIONING_SECONDS = 0.4
 CONFIG_CONDITIONING_SECONDS = 0.25   # per workload and reduction of the configs array, untimed
@@ -63,7 +69,39 @@ def _close(torch, got, want, reduction):
     return ok, float((err / (1e-5 + 2e-3 * want.abs())).max())   # worst error in units of the tolerance
 
 
-def run_configs(torch, fca, colreduce_ref, inputs, cores):
+def _c_abi_us(torch, qd, kd, red, causal, reps):
+    """The call through the C ABI with preallocated buffers (fcr_colreduce_to, fp32 result), `reps` times back to
+    back.  Returns (microseconds per call between two events on the stream, microseconds the host needs to
+    issue one call).  While the host is the faster of the two the first number is the time of the call's
+    kernels on the GPU."""
+    from flash_colreduce_amd import _lib
+    lib = _lib.load()
+    b, h, m, d = qd.shape
+    n = kd.shape[2]
+    out = torch.empty(b, h, n, device=qd.device, dtype=torch.float32)
+    lse = torch.empty(lib.fcr_lse_bytes(b, h, m, n, d) // 4, device=qd.device, dtype=torch.float32)
+    dt = {torch.float16: _lib.DTYPE_F16, torch.bfloat16: _lib.DTYPE_BF16, torch.float32: _lib.DTYPE_F32}[qd.dtype]
+    code = {"sum": _lib.REDUCE_SUM, "max": _lib.REDUCE_MAX, "mean": _lib.REDUCE_MEAN}[red]
+    qs, ks = _lib.strides4(qd.stride()), _lib.strides4(kd.stride())
+    stream = torch.cuda.current_stream(qd.device).cuda_stream
+    args = (qd.data_ptr(), kd.data_ptr(), out.data_ptr(), _lib.DTYPE_F32, lse.data_ptr(), dt, b, h, m, n, d, qs, ks,
+            1.0 / d ** 0.5, code, int(causal), stream)
+    call = lambda: lib.fcr_colreduce_to(*args)
+    for _ in range(3):
+        _lib.check(call())
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        call()
+    host = (time.perf_counter() - t0) / reps * 1e6
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / reps * 1e3, host
+
+
+def run_configs(torch, fca, colreduce_ref, inputs, cores, only=None):
     """The five named workloads.  GPU: flash_colreduce (fp32 result) timed with events; CPU: the oracle
     on a head sample, timed once (configs 4, 5) or best of three (1-3); parity on that sample."""
     dev = torch.device("cuda:0")
@@ -76,6 +114,8 @@ def run_configs(torch, fca, colreduce_ref, inputs, cores):
     ]
     out = []
     for name, make, causal, reductions, heads in specs:
+        if only is not None and int(name[-1]) not in only:
+            continue
         q, k = make()
         b, h, m, d = q.shape
         n = k.shape[2]
@@ -99,6 +139,7 @@ def run_configs(torch, fca, colreduce_ref, inputs, cores):
                     fn()
                 torch.cuda.synchronize()
             ms = _events_ms(torch, fn, reps)
+            kernel_us, host_us = _c_abi_us(torch, qd, kd, red, causal, max(reps, 50))
             cpu_s = None
             for _ in range(1 if flop > 1e11 else 3):
                 t0 = time.perf_counter()
@@ -106,7 +147,7 @@ def run_configs(torch, fca, colreduce_ref, inputs, cores):
                 dt = time.perf_counter() - t0
                 cpu_s = dt if cpu_s is None else min(cpu_s, dt)
             ok, worst = _close(torch, got[:, hs].cpu(), want, red)
-            r = {"ms": ms, "tflops": flop / (ms * 1e-3) / 1e12,
+            r = {"ms": ms, "kernel_us": kernel_us, "host_issue_us": host_us, "tflops": flop / (ms * 1e-3) / 1e12,
                  "frac_mfma_peak": flop / (ms * 1e-3) / 1e12 / PEAK_FP16_DENSE_TFLOPS,
                  "cpu_ms_per_call_extrapolated": cpu_s * 1e3 * h / len(hs),
                  "cpu_tflops": flop * len(hs) / h / cpu_s / 1e12, "pass": ok,
@@ -116,6 +157,7 @@ def run_configs(torch, fca, colreduce_ref, inputs, cores):
                 visible = sum(min(n, i + max(n - m, 0) + 1) for i in range(m)) / float(m * n)
                 r["tflops_visible_scores"] = 4.0 * b * h * m * n * d * visible / (ms * 1e-3) / 1e12
                 r["frac_hbm_peak"] = bytes_alg / (ms * 1e-3) / 1e12 / PEAK_HBM_TBPS
+                r["frac_hbm_peak_kernels"] = bytes_alg / (kernel_us * 1e-6) / 1e12 / PEAK_HBM_TBPS
             entry["reductions"][red] = r
         entry["pass"] = all(r["pass"] for r in entry["reductions"].values())
         out.append(entry)
@@ -132,6 +174,9 @@ def main():
     ap.add_argument("--cpu-heads", type=int, default=32,
                     help="heads of the workload the CPU oracle is timed on (0 = skip)")
     ap.add_argument("--no-configs", action="store_true", help="skip the five named workloads")
+    ap.add_argument("--configs", type=str, default=None, help="comma separated subset of the named workloads, e.g. 2,3")
+    ap.add_argument("--no-headline", action="store_true",
+                    help="skip the headline workload (value, roofline and cpu_baseline are then null); for profiler runs")
     ap.add_argument("--conditioning", type=float, default=CONDITIONING_SECONDS,
                     help="seconds of untimed calls before the warm-up (0 = none)")
     ap.add_argument("--copy-calib", action="store_true",
@@ -148,7 +193,7 @@ def main():
     import torch
     import flash_colreduce_amd as fca
     from flash_colreduce_amd import _lib
-    from tests import _inputs
+    from flash_colreduce_amd import workloads as _inputs
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible", file=sys.stderr)
@@ -156,6 +201,21 @@ def main():
     lib = _lib.load()
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    only = None if args.configs is None else {int(x) for x in args.configs.split(",") if x}
+    METRIC = ("effective TFLOP/s (4*B*H*M*N*D, halved for causal) of flash_colreduce sum, causal B1 H32 M=N=8192 "
+              "d128 fp16; one step = one fcr_colreduce call of the C ABI (both kernels, preallocated buffers, fp32 "
+              "result); the Python operator on the same tensors is ms_per_step_python_api")
+    if args.no_headline:
+        from oracle.colreduce_oracle import colreduce_ref
+        cores = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1)))
+        torch.set_num_threads(cores)
+        configs = run_configs(torch, fca, colreduce_ref, _inputs, cores, only)
+        print(json.dumps({"metric": METRIC, "value": None, "unit": "TFLOP/s", "n_gpus": 1, "steps": 0, "warmup": 0,
+                          "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "fp16",
+                          "data": "synthetic", "config": {"workload": "named workloads only (--no-headline)"},
+                          "roofline": None, "cpu_baseline": None, "configs": configs}), flush=True)
+        return
 
     B, H, M, N, D = 1, 32, 8192, 8192, 128
     q_cpu, k_cpu = _inputs.headline()
@@ -198,6 +258,13 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     ms_per_step_events = e0.elapsed_time(e1) / args.steps
+
+    # the reference's own call on the same tensors: torch allocations, both kernels, fp16 result
+    api = lambda: fca.flash_colreduce(q, k, "sum", is_causal=True)
+    for _ in range(args.warmup):
+        api()
+    torch.cuda.synchronize()
+    ms_per_step_python_api = _events_ms(torch, api, args.steps)
 
     reps = max(args.steps, 10)
     pass1()
@@ -250,13 +317,13 @@ def main():
     del q, k, out, lse
     torch.cuda.empty_cache()
 
-    configs = None if args.no_configs else run_configs(torch, fca, colreduce_ref, _inputs, cores)
+    configs = None if args.no_configs else run_configs(torch, fca, colreduce_ref, _inputs, cores, only)
 
     line = {
-        "metric": "effective TFLOP/s (4*B*H*M*N*D, halved for causal) of flash_colreduce sum, "
-                  "causal B1 H32 M=N=8192 d128 fp16",
+        "metric": METRIC,
         "value": value, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "ms_per_step_events": ms_per_step_events,
+        "ms_per_step_python_api": ms_per_step_python_api,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "fp16", "accumulate": "fp32", "data": "synthetic",
         "config": {"workload": "causal B=1 H=32 M=N=8192 D=128 fp16, reduction=sum, seed 0 N(0,1)",
