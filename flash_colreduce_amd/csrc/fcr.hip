@@ -19,6 +19,9 @@
 //                     their lse2) through LDS; writes out[bh, j] = sum_i or max_i 2^(s_ij-lse2_i).
 //   col_small_kernel  the same result for at most 128 query rows against many keys: queries resident
 //                     in every wave, keys streamed (HBM bound).
+//   col_fused_kernel  both sweeps in one for at most 128 query rows against many 16-bit keys: the scores of
+//                     1024 keys stay in registers while the workgroups that share a (batch, head) pair
+//                     exchange their row sums through tagged 64-bit slots, so the keys are read once.
 //   topk_mask_kernel  keep-mask of the k largest columns of every row of the result (one workgroup per
 //                     row; topk_spread_* kernels share a long row between workgroups).
 // where s_ij = scale * log2(e) * <q_i, k_j>.  The column kernels store the result type of the caller's choice

@@ -67,7 +67,7 @@ extern "C" {
 
 /* fcr_set_option */
 #define FCR_OPT_SINGLE_SWEEP 0 /* 0: few queries against many keys take the two kernels as well (default 1) */
-#define FCR_OPT_WAIT_POLLS 1   /* polls of a team's arrival counter after which a workgroup gives up (default 2^20) */
+#define FCR_OPT_WAIT_POLLS 1   /* polls of a team's slots after which a workgroup gives up (default 2^20) */
 
 /* size of the built-in scratch buffer of fcr_colreduce_static, per GPU */
 #define FCR_STATIC_SCRATCH_BYTES (16u << 20)
@@ -80,9 +80,10 @@ const char* fcr_last_error(void);
 
 /*
  * Bytes the lse buffer of fcr_row_lse / fcr_colreduce must have for a problem, whatever its dtype and
- * D.  The first B*H*M floats are the result; for few query rows and many keys the row kernel splits the
- * keys of a tile over several workgroups and keeps their partial results behind it.  0 for an empty
- * problem.
+ * D.  The first B*H*M floats are the result; scratch follows for few query rows against many keys: the
+ * partial results of the row kernel when it splits the keys of a tile over several workgroups, or the
+ * slots in which the workgroups of the single sweep publish their row sums (they depend on the number
+ * of compute units: call this with the operands' device current).  0 for an empty problem.
  */
 size_t fcr_lse_bytes(int B, int H, int M, int N, int D);
 
