@@ -50,6 +50,9 @@ def _declare(lib):
     lib.fcr_col_reduce_sum_max.argtypes = ([c.c_void_p] * 5 + common + [c.c_int, c.c_void_p])
     lib.fcr_topk_mask.restype = c.c_int
     lib.fcr_topk_mask.argtypes = [c.c_void_p, c.c_void_p, c.c_void_p, c.c_int64, c.c_int, c.c_int, c.c_void_p]
+    lib.fcr_topk_mask_typed.restype = c.c_int
+    lib.fcr_topk_mask_typed.argtypes = [c.c_void_p, c.c_int, c.c_void_p, c.c_void_p, c.c_int64, c.c_int, c.c_int,
+                                        c.c_void_p, c.c_size_t, c.c_void_p]
     lib.fcr_topk_bytes.restype = c.c_size_t
     lib.fcr_topk_bytes.argtypes = [c.c_int64, c.c_int]
     lib.fcr_topk_mask_ws.restype = c.c_int

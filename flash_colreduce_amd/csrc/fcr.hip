@@ -1743,7 +1743,25 @@ __global__ __launch_bounds__(256) void pack_f32_kernel(const float* __restrict__
 __device__ __forceinline__ uint32_t order_key(float x) {
   uint32_t b = __builtin_bit_cast(uint32_t, x);
   if (b == 0x80000000u) b = 0u;  // -0 and +0 are one value
+  if ((b & 0x7fffffffu) > 0x7f800000u) return 0xffffffffu;  // a NaN of either sign: one value above +inf (torch.topk's order)
   return b ^ ((uint32_t)((int32_t)b >> 31) | 0x80000000u);  // monotone in x for all non-NaN floats
+}
+
+// Score rows come as fp32, fp16 or bf16 (what the column kernels store); keys are taken from the widened
+// value, which is exact, so order and ties are those of the stored values.
+template <typename ET> __device__ __forceinline__ float widen(ET x) { return (float)x; }
+template <> __device__ __forceinline__ float widen<uint16_t>(uint16_t x) {   // bf16 bits
+  return __builtin_bit_cast(float, (uint32_t)x << 16);
+}
+// keys of the 4 elements at p, which is aligned to 4 elements
+template <typename ET> __device__ __forceinline__ void order_keys4(const ET* p, uint32_t* u) {
+  typedef ET ETx4 __attribute__((ext_vector_type(4)));
+  const ETx4 v = *reinterpret_cast<const ETx4*>(p);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) u[e] = order_key(widen<ET>(v[e]));
+}
+template <typename ET> __device__ __forceinline__ bool rows_aligned_to_4(const ET* scores, int N) {
+  return (N & 3) == 0 && (reinterpret_cast<uintptr_t>(scores) & (4 * sizeof(ET) - 1)) == 0;
 }
 __device__ __forceinline__ float key_value(uint32_t key) {
   return __builtin_bit_cast(float, (key & 0x80000000u) ? (key ^ 0x80000000u) : ~key);
@@ -1779,28 +1797,26 @@ __device__ __forceinline__ uint32_t ties_before(uint32_t mine, uint32_t* wave_eq
   return before;
 }
 
-template <int VPT>
-__global__ __launch_bounds__(kTopkThreads) void topk_mask_kernel(const float* __restrict__ scores,
+template <int VPT, typename ET>
+__global__ __launch_bounds__(kTopkThreads) void topk_mask_kernel(const ET* __restrict__ scores,
                                                                  uint8_t* __restrict__ mask,
                                                                  float* __restrict__ threshold, int N, int k) {
   constexpr int kW = kTopkThreads / 64;
   __shared__ uint32_t cnt[34];       // one counter per pass: nothing to reset between passes
   __shared__ uint32_t wave_eq[kW];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const float* s = scores + (int64_t)blockIdx.x * N;
+  const ET* s = scores + (int64_t)blockIdx.x * N;
   uint8_t* m = mask + (int64_t)blockIdx.x * N;
   const uint32_t kk = (uint32_t)min(max(k, 0), N);
   const int base = tid * VPT;
 
   uint32_t u[VPT];
-  // 16-byte loads when every row starts on a 16-byte boundary
-  if ((N & 3) == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0) {
+  // four elements per load when every row starts on such a boundary
+  if (rows_aligned_to_4(scores, N)) {
 #pragma unroll
     for (int i = 0; i < VPT; i += 4) {
       if (base + i < N) {
-        const f32x4 v = *reinterpret_cast<const f32x4*>(s + base + i);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) u[i + e] = order_key(v[e]);
+        order_keys4(s + base + i, u + i);
       } else {
 #pragma unroll
         for (int e = 0; e < 4; ++e) u[i + e] = 0u;   // padding: below every candidate (candidates are >= 1)
@@ -1808,7 +1824,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_mask_kernel(const float* __
     }
   } else {
 #pragma unroll
-    for (int i = 0; i < VPT; ++i) u[i] = (base + i < N) ? order_key(s[base + i]) : 0u;
+    for (int i = 0; i < VPT; ++i) u[i] = (base + i < N) ? order_key(widen<ET>(s[base + i])) : 0u;
   }
   if (tid < 34) cnt[tid] = 0;
   __syncthreads();
@@ -1879,7 +1895,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_mask_kernel(const float* __
   }
 }
 
-__global__ __launch_bounds__(kTopkThreads) void topk_mask_long_kernel(const float* __restrict__ scores,
+template <typename ET>
+__global__ __launch_bounds__(kTopkThreads) void topk_mask_long_kernel(const ET* __restrict__ scores,
                                                                       uint8_t* __restrict__ mask,
                                                                       float* __restrict__ threshold, int N, int k) {
   constexpr int kW = kTopkThreads / 64;
@@ -1887,7 +1904,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_mask_long_kernel(const floa
   __shared__ uint32_t sh_prefix, sh_need, sh_ties;
   __shared__ uint32_t wave_eq[kW];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const float* s = scores + (int64_t)blockIdx.x * N;
+  const ET* s = scores + (int64_t)blockIdx.x * N;
   uint8_t* m = mask + (int64_t)blockIdx.x * N;
   const uint32_t kk = (uint32_t)min(max(k, 0), N);
   uint32_t prefix = 0, decided = 0, need = kk;
@@ -1897,7 +1914,7 @@ __global__ __launch_bounds__(kTopkThreads) void topk_mask_long_kernel(const floa
     __syncthreads();
     for (int j0 = 0; j0 < N; j0 += kTopkThreads) {
       const int j = j0 + tid;
-      const uint32_t x = (j < N) ? order_key(s[j]) : 0u;
+      const uint32_t x = (j < N) ? order_key(widen<ET>(s[j])) : 0u;
       const bool live = (j < N) && ((x & decided) == prefix);
       const uint32_t d = (x >> shift) & 255u;
       const uint64_t lives = __builtin_amdgcn_ballot_w64(live);
@@ -1954,14 +1971,14 @@ __global__ __launch_bounds__(kTopkThreads) void topk_mask_long_kernel(const floa
   uint32_t before = 0;
   if (need < ties) {
     uint32_t mine = 0;
-    for (int i = 0; i < per; ++i) mine += (base + i < N && order_key(s[base + i]) == T) ? 1u : 0u;
+    for (int i = 0; i < per; ++i) mine += (base + i < N && order_key(widen<ET>(s[base + i])) == T) ? 1u : 0u;
     before = ties_before(mine, wave_eq, lane, wave);
   }
   const bool keep_all_ties = need >= ties;
   for (int i = 0; i < per; ++i) {
     const int j = base + i;
     if (j >= N) break;
-    const uint32_t x = order_key(s[j]);
+    const uint32_t x = order_key(widen<ET>(s[j]));
     const bool eq = x == T;
     m[j] = ((kk > 0) && ((x > T) || (eq && (keep_all_ties || before < need)))) ? 1 : 0;
     if (eq) ++before;
@@ -2027,29 +2044,25 @@ __device__ __forceinline__ TopkState topk_choose(const uint32_t* __restrict__ hi
 }
 
 // The VPT keys of a thread from column col0 on; columns past N get key 0 and valid bit 0.
-template <int VPT>
-__device__ __forceinline__ uint32_t topk_load(const float* __restrict__ s, int N, int col0, bool vec, uint32_t u[VPT]) {
+template <int VPT, typename ET>
+__device__ __forceinline__ uint32_t topk_load(const ET* __restrict__ s, int N, int col0, bool vec, uint32_t u[VPT]) {
   if (vec && col0 + VPT <= N) {
 #pragma unroll
-    for (int i = 0; i < VPT; i += 4) {
-      const f32x4 a = *reinterpret_cast<const f32x4*>(s + col0 + i);
-#pragma unroll
-      for (int e = 0; e < 4; ++e) u[i + e] = order_key(a[e]);
-    }
+    for (int i = 0; i < VPT; i += 4) order_keys4(s + col0 + i, u + i);
     return VPT == 32 ? 0xffffffffu : (1u << (VPT & 31)) - 1u;
   }
   uint32_t valid = 0;
 #pragma unroll
   for (int i = 0; i < VPT; ++i) {
     const bool in = col0 + i < N;
-    u[i] = in ? order_key(s[in ? col0 + i : 0]) : 0u;
+    u[i] = in ? order_key(widen<ET>(s[in ? col0 + i : 0])) : 0u;
     valid |= in ? (1u << i) : 0u;
   }
   return valid;
 }
 
-template <int PASS, int VPT>
-__global__ __launch_bounds__(kTopkThreads) void topk_spread_hist_kernel(const float* __restrict__ scores,
+template <int PASS, int VPT, typename ET>
+__global__ __launch_bounds__(kTopkThreads) void topk_spread_hist_kernel(const ET* __restrict__ scores,
                                                                         uint32_t* __restrict__ ws, int64_t rows,
                                                                         int N, int k, int parts) {
   __shared__ uint32_t bins[256];
@@ -2063,8 +2076,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_spread_hist_kernel(const fl
   uint32_t* mine = ws + (PASS & 1) * words + ((size_t)row * parts + part) * 256;
 
   uint32_t u[VPT];
-  const float* s = scores + row * N;
-  const bool vec = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0;
+  const ET* s = scores + row * N;
+  const bool vec = rows_aligned_to_4(scores, N);
   const uint32_t valid = topk_load<VPT>(s, N, (part * kTopkThreads + tid) * VPT, vec, u);
 
   TopkState st{0u, (uint32_t)min(max(k, 0), N), 0u, 0u};
@@ -2095,8 +2108,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_spread_hist_kernel(const fl
   if (tid < 256) mine[tid] = hist[tid];
 }
 
-template <int VPT>
-__global__ __launch_bounds__(kTopkThreads) void topk_spread_write_kernel(const float* __restrict__ scores,
+template <int VPT, typename ET>
+__global__ __launch_bounds__(kTopkThreads) void topk_spread_write_kernel(const ET* __restrict__ scores,
                                                                          uint8_t* __restrict__ mask,
                                                                          float* __restrict__ threshold,
                                                                          const uint32_t* __restrict__ ws, int64_t rows,
@@ -2113,8 +2126,8 @@ __global__ __launch_bounds__(kTopkThreads) void topk_spread_write_kernel(const f
   const uint32_t* last = ws + words + (size_t)row * parts * 256;   // the histograms of digit 3 (3 & 1 == 1)
 
   uint32_t u[VPT];
-  const float* s = scores + row * N;
-  const bool vec = (N & 3) == 0 && (reinterpret_cast<uintptr_t>(scores) & 15) == 0;
+  const ET* s = scores + row * N;
+  const bool vec = rows_aligned_to_4(scores, N);
   const int col0 = (part * kTopkThreads + tid) * VPT;
   const uint32_t valid = topk_load<VPT>(s, N, col0, vec, u);
 
@@ -2498,16 +2511,38 @@ void launch_sweeps(int dtype, int which, const Params& p, int ksteps, bool causa
   else fcr_detail::sweeps_f32_long_rows(which, p, ksteps, causal, mode, s);
 }
 
-template <int VPT>
-void launch_topk_spread(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, uint32_t* w,
+template <int VPT, typename ET>
+void launch_topk_spread(const ET* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, uint32_t* w,
                         hipStream_t s) {
   const int parts = (N + VPT * kTopkThreads - 1) / (VPT * kTopkThreads);
   const dim3 grid((unsigned)(rows * parts)), block(kTopkThreads);
-  hipLaunchKernelGGL((topk_spread_hist_kernel<0, VPT>), grid, block, 0, s, scores, w, rows, N, k, parts);
-  hipLaunchKernelGGL((topk_spread_hist_kernel<1, VPT>), grid, block, 0, s, scores, w, rows, N, k, parts);
-  hipLaunchKernelGGL((topk_spread_hist_kernel<2, VPT>), grid, block, 0, s, scores, w, rows, N, k, parts);
-  hipLaunchKernelGGL((topk_spread_hist_kernel<3, VPT>), grid, block, 0, s, scores, w, rows, N, k, parts);
-  hipLaunchKernelGGL((topk_spread_write_kernel<VPT>), grid, block, 0, s, scores, mask, threshold, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_hist_kernel<0, VPT, ET>), grid, block, 0, s, scores, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_hist_kernel<1, VPT, ET>), grid, block, 0, s, scores, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_hist_kernel<2, VPT, ET>), grid, block, 0, s, scores, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_hist_kernel<3, VPT, ET>), grid, block, 0, s, scores, w, rows, N, k, parts);
+  hipLaunchKernelGGL((topk_spread_write_kernel<VPT, ET>), grid, block, 0, s, scores, mask, threshold, w, rows, N, k,
+                     parts);
+}
+
+// The top-k launches for one element type: spread over workgroups when the caller brought enough scratch
+// for a long row, else one workgroup per row.
+template <typename ET>
+int topk_any(const ET* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* ws, size_t ws_bytes,
+             hipStream_t s) {
+  const size_t want = fcr_topk_bytes(rows, N);
+  if (ws && want != 0 && ws_bytes >= want) {
+    uint32_t* w = static_cast<uint32_t*>(ws);
+    // 32 keys per thread while that leaves a workgroup per CU, else 8
+    const int64_t coarse = rows * ((N + 32 * kTopkThreads - 1) / (32 * kTopkThreads));
+    if (coarse >= chip_cus()) launch_topk_spread<32>(scores, mask, threshold, rows, N, k, w, s);
+    else launch_topk_spread<8>(scores, mask, threshold, rows, N, k, w, s);
+    return 0;
+  }
+  const dim3 grid((unsigned)rows), block(kTopkThreads);
+  if (N <= 8 * kTopkThreads) hipLaunchKernelGGL((topk_mask_kernel<8, ET>), grid, block, 0, s, scores, mask, threshold, N, k);
+  else if (N <= 32 * kTopkThreads) hipLaunchKernelGGL((topk_mask_kernel<32, ET>), grid, block, 0, s, scores, mask, threshold, N, k);
+  else hipLaunchKernelGGL(topk_mask_long_kernel<ET>, grid, block, 0, s, scores, mask, threshold, N, k);
+  return 0;
 }
 }  // namespace
 
@@ -2650,31 +2685,29 @@ size_t fcr_topk_bytes(int64_t rows, int N) {
   return 2 * topk_hist_words(rows, parts) * sizeof(uint32_t) + (size_t)rows * 4 * sizeof(TopkState);
 }
 
+int fcr_topk_mask_typed(const void* scores, int dtype, uint8_t* mask, float* threshold, int64_t rows, int N, int k,
+                        void* ws, size_t ws_bytes, void* stream) {
+  if (!scores || !mask) return fail(FCR_E_NULL, "null pointer argument");
+  if (dtype != FCR_DTYPE_F16 && dtype != FCR_DTYPE_BF16 && dtype != FCR_DTYPE_F32)
+    return fail(FCR_E_DTYPE, "scores must be fp16, bf16 or fp32");
+  // one workgroup of 1024 threads per row (or per part of a row), fewer than 2^32 threads per launch
+  if (rows < 1 || rows >= (1ll << 22) || N < 1) return fail(FCR_E_SHAPE, "rows must be in [1, 2^22) and N >= 1");
+  if (ws && (reinterpret_cast<uintptr_t>(ws) & 15) != 0)
+    return fail(FCR_E_STRIDE, "the top-k workspace must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (dtype == FCR_DTYPE_F32) topk_any(static_cast<const float*>(scores), mask, threshold, rows, N, k, ws, ws_bytes, s);
+  else if (dtype == FCR_DTYPE_F16) topk_any(static_cast<const _Float16*>(scores), mask, threshold, rows, N, k, ws, ws_bytes, s);
+  else topk_any(static_cast<const uint16_t*>(scores), mask, threshold, rows, N, k, ws, ws_bytes, s);
+  return launched("top-k kernels");
+}
+
 int fcr_topk_mask_ws(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* ws,
                      size_t ws_bytes, void* stream) {
-  const size_t want = fcr_topk_bytes(rows, N);
-  if (!ws || want == 0 || ws_bytes < want) return fcr_topk_mask(scores, mask, threshold, rows, N, k, stream);
-  if (!scores || !mask) return fail(FCR_E_NULL, "null pointer argument");
-  if ((reinterpret_cast<uintptr_t>(ws) & 15) != 0) return fail(FCR_E_STRIDE, "the top-k workspace must be 16-byte aligned");
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  uint32_t* w = static_cast<uint32_t*>(ws);
-  // 32 keys per thread while that leaves a workgroup per CU, else 8
-  const int64_t coarse = rows * ((N + 32 * kTopkThreads - 1) / (32 * kTopkThreads));
-  if (coarse >= chip_cus()) launch_topk_spread<32>(scores, mask, threshold, rows, N, k, w, s);
-  else launch_topk_spread<8>(scores, mask, threshold, rows, N, k, w, s);
-  return launched("topk_spread kernels");
+  return fcr_topk_mask_typed(scores, FCR_DTYPE_F32, mask, threshold, rows, N, k, ws, ws_bytes, stream);
 }
 
 int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream) {
-  if (!scores || !mask) return fail(FCR_E_NULL, "null pointer argument");
-  // one workgroup of 1024 threads per row, fewer than 2^32 threads per launch
-  if (rows < 1 || rows >= (1ll << 22) || N < 1) return fail(FCR_E_SHAPE, "rows must be in [1, 2^22) and N >= 1");
-  const dim3 grid((unsigned)rows), block(kTopkThreads);
-  hipStream_t s = static_cast<hipStream_t>(stream);
-  if (N <= 8 * kTopkThreads) hipLaunchKernelGGL(topk_mask_kernel<8>, grid, block, 0, s, scores, mask, threshold, N, k);
-  else if (N <= 32 * kTopkThreads) hipLaunchKernelGGL(topk_mask_kernel<32>, grid, block, 0, s, scores, mask, threshold, N, k);
-  else hipLaunchKernelGGL(topk_mask_long_kernel, grid, block, 0, s, scores, mask, threshold, N, k);
-  return launched("topk_mask_kernel");
+  return fcr_topk_mask_typed(scores, FCR_DTYPE_F32, mask, threshold, rows, N, k, nullptr, 0, stream);
 }
 
 int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, int is_key, void* stream) {

@@ -293,7 +293,8 @@ def row_lse2(query: torch.Tensor, key: torch.Tensor, is_causal: bool = False,
 
 
 def topk_keep_mask(scores: torch.Tensor, k: int, return_threshold: bool = False):
-    """Boolean mask of the k largest entries along the last dimension (ties: lower index wins).
+    """Boolean mask of the k largest entries along the last dimension (ties: lower index wins; a NaN
+    ranks above +inf, as in torch.topk).
 
     The step a pruning caller takes on the (B, H, N) result of flash_colreduce; not part of the
     reference's package.  `scores` is a float32, float16 or bfloat16 GPU tensor; the result has its shape.
@@ -304,9 +305,7 @@ def topk_keep_mask(scores: torch.Tensor, k: int, return_threshold: bool = False)
     if scores.dtype not in _DTYPES or scores.dim() < 1:
         raise ValueError(f"scores must be a float32, float16 or bfloat16 tensor with at least one dimension. "
                          f"Got {scores.dtype}.")
-    # 16-bit scores (what flash_colreduce returns for 16-bit operands) are widened first: exact, so the
-    # order and the ties are those of the 16-bit values
-    s = scores.contiguous() if scores.dtype == torch.float32 else scores.float().contiguous()
+    s = scores.contiguous()   # 16-bit scores (what flash_colreduce returns for 16-bit operands) are read as they are
     n = s.shape[-1]
     rows = s.numel() // n if n else 0
     if rows > 0 and n > 0:
@@ -319,7 +318,8 @@ def topk_keep_mask(scores: torch.Tensor, k: int, return_threshold: bool = False)
         nbytes = lib.fcr_topk_bytes(rows, n)   # > 0 for long rows: scratch that lets workgroups share a row
         ws = torch.empty(nbytes, device=s.device, dtype=torch.uint8) if nbytes else None
         with torch.cuda.device(s.device):
-            _lib.check(lib.fcr_topk_mask_ws(s.data_ptr(), mask.data_ptr(), thr.data_ptr() if thr is not None else None,
-                                            rows, n, int(k), ws.data_ptr() if ws is not None else None, nbytes,
-                                            torch.cuda.current_stream(s.device).cuda_stream))
+            _lib.check(lib.fcr_topk_mask_typed(s.data_ptr(), _DTYPES[s.dtype], mask.data_ptr(),
+                                               thr.data_ptr() if thr is not None else None, rows, n, int(k),
+                                               ws.data_ptr() if ws is not None else None, nbytes,
+                                               torch.cuda.current_stream(s.device).cuda_stream))
     return (mask, thr) if return_threshold else mask

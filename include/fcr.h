@@ -121,7 +121,8 @@ int fcr_col_reduce_sum_max(const void* q, const void* k, const float* lse, float
  * the calls above): mask[r, j] = 1 for exactly min(max(k,0), N) columns of row r, 0 elsewhere; among
  * equal values the lower column wins.  threshold (optional, may be NULL) receives the k-th largest
  * value of each row.  No counterpart in the reference: it is the step its pruning callers take on
- * the reduced columns (README.md:9).  NaNs are not ordered.
+ * the reduced columns (README.md:9).  A NaN of either sign ranks above +inf (the order of torch.topk),
+ * NaNs tie with each other; -0 and +0 are one value.  A threshold that is a NaN is stored as a NaN.
  */
 int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* stream);
 
@@ -135,6 +136,14 @@ int fcr_topk_mask(const float* scores, uint8_t* mask, float* threshold, int64_t 
 size_t fcr_topk_bytes(int64_t rows, int N);
 int fcr_topk_mask_ws(const float* scores, uint8_t* mask, float* threshold, int64_t rows, int N, int k, void* ws,
                      size_t ws_bytes, void* stream);
+
+/*
+ * The same for score rows of any FCR_DTYPE_* element type: fp16 and bf16 rows, as fcr_colreduce_to stores
+ * them for 16-bit operands, are read as they are (order and ties of the stored values; threshold stays
+ * fp32).  ws may be NULL (then ws_bytes is ignored); fcr_topk_bytes does not depend on the type.
+ */
+int fcr_topk_mask_typed(const void* scores, int dtype, uint8_t* mask, float* threshold, int64_t rows, int N, int k,
+                        void* ws, size_t ws_bytes, void* stream);
 
 /*
  * A faster and less exact alternative to FCR_DTYPE_F32 for fp32 operands whose values fit fp16 (the

@@ -196,8 +196,10 @@ def row_lse2_ref(q: torch.Tensor, k: torch.Tensor, is_causal: bool = False,
 
 def topk_mask_ref(scores, k: int) -> np.ndarray:
     """Keep-mask of the k largest entries of every row of a 2-D array; among equal values the lower
-    column wins.  Pinned by its defining properties (tests/test_oracle.py::test_topk_mask_ref): exactly
-    min(max(k,0),N) kept, every kept value >= every dropped one, kept ties precede dropped ties.
+    column wins; a NaN ranks above +inf and NaNs tie with each other (the order torch.topk uses).
+    Pinned by its defining properties (tests/test_oracle.py::test_topk_mask_ref): exactly
+    min(max(k,0),N) kept, every kept value >= every dropped one, kept ties precede dropped ties; and
+    against torch.topk on rows with NaNs.
     The reference has no such function; its callers do this step themselves (README.md:9)."""
     a = np.asarray(scores)
     rows, n = a.shape
@@ -205,6 +207,9 @@ def topk_mask_ref(scores, k: int) -> np.ndarray:
     mask = np.zeros((rows, n), dtype=bool)
     cols = np.arange(n)
     for r in range(rows):
-        order = np.lexsort((cols, -a[r].astype(np.float64)))  # by value descending, then column ascending
+        v = a[r].astype(np.float64)
+        nan = np.isnan(v)
+        # NaNs first, then by value descending, then column ascending
+        order = np.lexsort((cols, np.where(nan, 0.0, -v), ~nan))
         mask[r, order[:kk]] = True
     return mask

@@ -200,6 +200,32 @@ def test_topk_mask_ref():
             assert kept_ties == list(tie_cols[:len(kept_ties)])
 
 
+def test_topk_mask_ref_with_nans():
+    """NaNs rank above +inf and tie with each other: hand cases, then torch.topk (which orders NaNs the
+    same way) on rows of distinct values with NaNs of both signs."""
+    import torch
+    from oracle.colreduce_oracle import topk_mask_ref
+    nan, inf = float("nan"), float("inf")
+    a = np.array([[1.0, nan, inf, -inf, nan, 2.0]])
+    np.testing.assert_array_equal(topk_mask_ref(a, 1), [[0, 1, 0, 0, 0, 0]])
+    np.testing.assert_array_equal(topk_mask_ref(a, 2), [[0, 1, 0, 0, 1, 0]])
+    np.testing.assert_array_equal(topk_mask_ref(a, 3), [[0, 1, 1, 0, 1, 0]])
+    np.testing.assert_array_equal(topk_mask_ref(a, 5), [[1, 1, 1, 0, 1, 1]])
+    g = torch.Generator().manual_seed(3)
+    v = torch.randperm(300, generator=g).float().view(3, 100) - 150.0    # distinct values
+    v[0, [3, 50, 77]] = nan
+    v[1, 9] = -nan
+    v[2, 5] = inf
+    v[2, 6] = nan
+    for k in (1, 2, 3, 4, 10, 99):
+        want = torch.zeros(3, 100, dtype=torch.bool)
+        want.scatter_(1, torch.topk(v, k, dim=1).indices, True)
+        if k >= 3:    # fewer than the NaNs of row 0: torch may pick any of them, the oracle the first
+            np.testing.assert_array_equal(topk_mask_ref(v.numpy(), k), want.numpy())
+        else:
+            np.testing.assert_array_equal(topk_mask_ref(v.numpy(), k)[1:], want.numpy()[1:])
+
+
 def test_bad_reduction():
     q, k = _rand(1, 1, 2, 2, 2)
     with pytest.raises(ValueError, match="Invalid reduction"):

@@ -178,7 +178,7 @@ def test_config5_full_size():
 
 def test_headline_shape_fp16():
     q, k = _inputs.headline()
-    _full_size(q, k, ["sum"], [5], "headline")
+    _full_size(q, k, ["sum"], [0, 5, 18, 31], "headline")
 
 
 # --- beyond the reference's grid ----------------------------------------------------------------
@@ -584,7 +584,7 @@ def test_nan_and_inf_inputs(causal):
     hidden entries of a NaN row NaN as well, naive.py:24-25; its kernel, like this one, never visits
     them, flash.py:198-207), as are rows and (b,h) pairs without one.  The column maximum follows IEEE
     maxNum (a NaN operand is dropped, like the Triton max at flash.py:123-124), so 'max' is compared on
-    the columns no NaN row sees."""
+    the columns no NaN row sees (test_max_leaves_nan_rows_out checks it on the others)."""
     b, h, m, n, d = 1, 4, 150, 260, 64
     q, k = _inputs.randn_pair(b, h, m, n, d, seed=55)
     q = q.clone()
@@ -611,6 +611,44 @@ def test_nan_and_inf_inputs(causal):
         if causal:
             assert ok[0, 0].any() and ok[0, 1].any()
         check(got[ok], want[ok], red, f"columns no NaN row sees, causal={causal}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n", [(150, 260), (300, 3000), (64, 700), (100, 900), (64, 2048), (128, 4096)])
+def test_max_leaves_nan_rows_out(m, n, causal):
+    """The column maximum of a column that a NaN row sees is the maximum over the other rows that see it,
+    and 0 when there is none: a NaN is dropped by the maximum (IEEE maxNum), as in the reference's kernel
+    (tl.max and tl.atomic_max, flash.py:123-124,262-273), not propagated as by the materialising reference
+    (naive.py:36-37).  Every column kernel (resident keys, streamed keys, single sweep, sum and max from
+    one sweep), checked ON the columns the NaN rows see, against a float64 softmax written out here."""
+    b, h, d = 1, 3, 64
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=77 + m)
+    q, k = q.half().clone(), k.half().clone()
+    q[0, 0, m // 2, 5] = float("nan")       # head 0: one NaN row in the middle
+    q[0, 1, m - 1, 0] = float("nan")        # head 1: the last row, the only one that sees the last column when causal
+    q[0, 1, 3, 1] = float("inf")            #         and a row with +inf and -inf scores
+    k[0, 2, n - 5, 7] = float("-inf")       # head 2: a key that gives +inf, -inf scores
+    c = max(n - m, 0)
+    vis = (torch.arange(m)[:, None] + c >= torch.arange(n)[None, :]) if causal else torch.ones(m, n, dtype=torch.bool)
+    s = torch.einsum("bhmd,bhnd->bhmn", q.double(), k.double()) / math.sqrt(d)
+    s = torch.where(vis, s, torch.full_like(s, float("-inf")))
+    bad = (torch.isnan(s) | (s == float("inf"))).any(-1)                     # [b, h, m]
+    p = torch.softmax(torch.where(bad[..., None], torch.zeros_like(s), s), dim=-1)
+    p = torch.where(vis, p, torch.zeros_like(p))
+    want_max = torch.where(bad[..., None], torch.zeros_like(p), p).amax(-2)
+    nan_cols = (bad[..., None] & vis).any(-2)
+    want_sum = torch.where(nan_cols, torch.full_like(want_max, float("nan")),
+                           torch.where(bad[..., None], torch.zeros_like(p), p).sum(-2))
+    assert bad[0, 0].sum() == 1 and bad[0, 1].sum() == 2 and bad[0, 2].sum() >= 1
+    if causal:
+        assert want_max[0, 1, -1] == 0    # no row left for the last column
+    qd, kd = q.cuda(), k.cuda()
+    got = fca.flash_colreduce(qd, kd, "max", is_causal=causal, out_dtype=torch.float32).cpu()
+    assert not torch.isnan(got).any()
+    torch.testing.assert_close(got.double(), want_max, rtol=2e-3, atol=1e-30)
+    both_sum, both_max = fca.flash_colreduce_multi(qd, kd, ["sum", "max"], is_causal=causal, out_dtype=torch.float32)
+    torch.testing.assert_close(both_max.cpu().double(), want_max, rtol=2e-3, atol=1e-30)
+    torch.testing.assert_close(both_sum.cpu().double(), want_sum, rtol=2e-3, atol=1e-5, equal_nan=True)
 
 
 def test_heavy_hitter_columns_small():
@@ -792,6 +830,52 @@ def test_topk_takes_the_operator_result_as_it_comes():
     assert (mask.view(3, 3000).cpu().numpy() == want).all()
     with pytest.raises(ValueError):
         fca.topk_keep_mask(scores.to(torch.float64), 5)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n,k", [(1, 1), (7, 3), (1000, 100), (1027, 1000), (8192, 2048), (8190, 17), (32768, 5000),
+                                 (32770, 300), (70001, 20000), (300004, 1000)])
+def test_topk_reads_16_bit_rows(n, k, dtype):
+    """16-bit score rows are read by the kernels themselves (every kernel of the selection, rows that do and
+    do not start on 8-byte boundaries): heavy ties, as 16-bit values have them, against the oracle on the
+    widened values; the threshold is the k-th largest value, widened."""
+    from oracle.colreduce_oracle import topk_mask_ref
+    g = torch.Generator().manual_seed(7 * n + k)
+    vals = torch.randn(5, n, generator=g).to(dtype)
+    vals[1] = (torch.rand(n, generator=g) * 4).to(dtype)          # a few hundred distinct values
+    vals[2] = 0.5
+    vals[3, ::2] = -0.0
+    vals[3, 1::2] = 0.0
+    mask, thr = fca.topk_keep_mask(vals.cuda(), k, return_threshold=True)
+    want = topk_mask_ref(vals.float().numpy(), k)
+    assert (mask.cpu().numpy() == want).all()
+    kth = torch.sort(vals.float(), dim=1, descending=True).values[:, k - 1]
+    assert thr.dtype == torch.float32 and torch.equal(thr.cpu() + 0.0, kth + 0.0)   # + 0.0: -0 and +0 are one value
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n", [100, 5000, 20000, 40000, 70001])
+def test_topk_orders_nans_above_everything(n, dtype):
+    """A NaN of either sign ranks above +inf, NaNs tie (lower column first): every kernel of the selection
+    against the oracle; the threshold is a NaN exactly when the k-th largest entry is one."""
+    from oracle.colreduce_oracle import topk_mask_ref
+    g = torch.Generator().manual_seed(n)
+    vals = torch.randn(4, n, generator=g).to(dtype)
+    nan = float("nan")
+    vals[0, [3, n // 2, n - 1]] = nan
+    vals[0, 7] = float("inf")
+    vals[1, 5] = -nan
+    vals[1, 50] = nan
+    vals[2, ::3] = nan                                   # a third of the row
+    vals[3] = nan                                        # the whole row
+    vals[3, 10] = 1.0
+    lib_rows = vals.cuda()
+    for k in (1, 2, 3, 4, 5, n // 3, n // 2, n - 1, n):
+        mask, thr = fca.topk_keep_mask(lib_rows, k, return_threshold=True)
+        want = topk_mask_ref(vals.float().numpy(), k)
+        assert (mask.cpu().numpy() == want).all(), k
+        nans = torch.isnan(vals.float()).sum(1)
+        assert torch.equal(torch.isnan(thr.cpu()), nans >= k), k
 
 
 def test_topk_on_reduced_columns():
