@@ -1,6 +1,7 @@
 """Latency / peak-memory sweep over the reference's 20 benchmark shapes.
 
     python -m flash_colreduce_amd.benchmark [--budget SECONDS] [--no-naive] [--rows 0,13] [--dtype fp16|bf16|fp32] [--out FILE]
+    python -m flash_colreduce_amd.benchmark --shape 1,32,8192,8192,128,1 [--constant]     (one shape B,H,M,N,D,causal)
     python -m flash_colreduce_amd.benchmark --topk
 
 Same shapes and method as the reference's harness (benchmarks/run.py:11-92): fp16, H = 32, D = 128,
@@ -60,7 +61,8 @@ def measure_memory(fn) -> float:
 DTYPES = {"fp16": torch.float16, "bf16": torch.bfloat16, "fp32": torch.float32}
 
 
-def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None, dtype: str = "fp16"):
+def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None, dtype: str = "fp16", shapes=CONFIGS,
+        constant: bool = False):
     name = torch.cuda.get_device_name(0)
     print(f"Benchmark results on {name} ({dtype}, reduction=sum)", file=out)
     head = (f"{'configuration':<48} {'flash ms':>10} {'naive ms':>10} {'speedup':>8} {'flash MB':>10} "
@@ -69,13 +71,16 @@ def run(budget: float = 2.0, with_naive: bool = True, out=sys.stdout, only=None,
     print("-" * len(head), file=out)
     rows = []
     with torch.inference_mode():
-        for index, cfg in enumerate(CONFIGS):
+        for index, cfg in enumerate(shapes):
             if only is not None and index not in only:
                 continue
             b, h, m, n, d, causal = (cfg[k] for k in ("b", "h", "m", "n", "d", "is_causal"))
             g = torch.Generator(device="cuda").manual_seed(0)
             q = torch.randn(b, h, m, d, device="cuda", dtype=DTYPES[dtype], generator=g)
             k = torch.randn(b, h, n, d, device="cuda", dtype=DTYPES[dtype], generator=g)
+            if constant:   # every element 0.5: the same instructions on operands that toggle no bits
+                q.fill_(0.5)
+                k.fill_(0.5)
             flash = lambda: flash_colreduce(q, k, reduction="sum", is_causal=causal)  # noqa: E731
             naive = lambda: naive_colreduce(q, k, reduction="sum", is_causal=causal)  # noqa: E731
             f_ms, f_mb = measure_latency(flash, budget), measure_memory(flash)
@@ -140,6 +145,9 @@ def main():
     ap.add_argument("--out", default=None, help="also write the table to this file")
     ap.add_argument("--dtype", default="fp16", choices=sorted(DTYPES), help="element type of q and k (the reference's table is fp16)")
     ap.add_argument("--topk", action="store_true", help="time the top-k keep-mask against torch.topk instead")
+    ap.add_argument("--shape", default=None, help="B,H,M,N,D,causal (0 or 1): this one shape instead of the table")
+    ap.add_argument("--constant", action="store_true",
+                    help="operands filled with 0.5 instead of N(0,1) draws (the clock the GPU keeps depends on the data)")
     args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("benchmark needs a GPU")
@@ -147,12 +155,17 @@ def main():
         run_topk()
         return
     only = None if args.rows is None else {int(r) for r in args.rows.split(",")}
+    shapes = CONFIGS
+    if args.shape:
+        b, h, m, n, d, causal = (int(x) for x in args.shape.split(","))
+        shapes, only = [dict(b=b, h=h, m=m, n=n, d=d, is_causal=bool(causal))], None
+    kw = dict(only=only, dtype=args.dtype, shapes=shapes, constant=args.constant)
     if args.out:
         with open(args.out, "w") as f:
-            run(args.budget, not args.no_naive, out=f, only=only, dtype=args.dtype)
+            run(args.budget, not args.no_naive, out=f, **kw)
         print(open(args.out).read())
     else:
-        run(args.budget, not args.no_naive, only=only, dtype=args.dtype)
+        run(args.budget, not args.no_naive, **kw)
 
 
 if __name__ == "__main__":

@@ -43,7 +43,8 @@
 
 // The file can be compiled whole, or in parts that are linked together (the build script does that to
 // use several cores): part 0 holds the C ABI and the small kernels, parts 1-4 the sweeps of one element
-// type each (fp16, bf16, fp32 rows up to 512 bytes, longer fp32 rows).
+// type each (fp16, bf16, fp32 rows up to 512 bytes, longer fp32 rows), parts 5 and 6 the sweeps over fp16 and
+// bf16 rows of more than 512 bytes.
 #ifndef FCR_PART
 #define FCR_PART -1
 #endif
@@ -84,6 +85,8 @@ void sweeps_f16(int which, const Params& p, int ksteps, bool causal, int mode, h
 void sweeps_bf16(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_f32(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_f32_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
+void sweeps_f16_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
+void sweeps_bf16_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 extern thread_local bool fused_refused;   // set by a launcher of col_fused_kernel that did not launch
 }  // namespace fcr_detail
 
@@ -149,8 +152,8 @@ inline int row_blocks_per_wave(int ksteps, int M, int N, int64_t bh, bool causal
 inline int row_tile_rows(int ksteps, int M, int N, int64_t bh, bool causal) {
   return kWaves * 32 * row_blocks_per_wave(ksteps, M, N, bh, causal);
 }
-constexpr int kMaxKSteps = 8;                 // 16-bit elements: D <= 256
-constexpr int kMaxKStepsF32 = 16;             // fp32: D <= 256 as well (rows of up to 1 KiB, one workgroup per CU)
+constexpr int kMaxKSteps = 8;                 // rows of up to 512 bytes: two workgroups per CU
+constexpr int kMaxKStepsF32 = 16;             // rows of up to 1 KiB (fp32: D <= 256, 16-bit elements: D <= 512), one workgroup per CU
 constexpr int kChunk = 64;                    // streamed rows per LDS stage (two 32-row sub-steps)
 constexpr int64_t kMaxWorkgroups = 1ll << 24; // the runtime refuses launches of 2^32 threads or more
 constexpr float kNegInf = -__builtin_inff();
@@ -2230,8 +2233,8 @@ int make_params(Params& p, const void* q, const void* k, int dtype, int B, int H
     return fail(FCR_E_DTYPE, "dtype must be FCR_DTYPE_F16, FCR_DTYPE_BF16 or FCR_DTYPE_F32");
   if (B < 1 || H < 1 || M < 1 || N < 1) return fail(FCR_E_SHAPE, "B, H, M, N must be >= 1");
   const int esize = elem_bytes(dtype);
-  if (D < 1 || D > 256 || (D * esize) % 16 != 0)
-    return fail(FCR_E_SHAPE, esize == 2 ? "D must be a multiple of 8 in [8, 256]"
+  if (D < 1 || D * esize > 64 * kMaxKStepsF32 || (D * esize) % 16 != 0)
+    return fail(FCR_E_SHAPE, esize == 2 ? "D must be a multiple of 8 in [8, 512]"
                                          : "D must be a multiple of 4 in [4, 256] for FCR_DTYPE_F32");
   if (M > (1 << 30) || N > (1 << 30)) return fail(FCR_E_SHAPE, "M and N must be <= 2^30");
   const int64_t bh = (int64_t)B * H;
@@ -2440,17 +2443,17 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
     default: CALL(DT, 8); break;                           \
   }
 
-// fp32 rows of more than 512 bytes: 9 to 16 k-steps
-#define FCR_DISPATCH_KS_F32_LONG(ksteps, CALL)                    \
-  switch (ksteps) {                                               \
-    case 9: CALL(FCR_DTYPE_F32, 9); break;                        \
-    case 10: CALL(FCR_DTYPE_F32, 10); break;                      \
-    case 11: CALL(FCR_DTYPE_F32, 11); break;                      \
-    case 12: CALL(FCR_DTYPE_F32, 12); break;                      \
-    case 13: CALL(FCR_DTYPE_F32, 13); break;                      \
-    case 14: CALL(FCR_DTYPE_F32, 14); break;                      \
-    case 15: CALL(FCR_DTYPE_F32, 15); break;                      \
-    default: CALL(FCR_DTYPE_F32, 16); break;                      \
+// rows of more than 512 bytes: 9 to 16 k-steps
+#define FCR_DISPATCH_KS_LONG(DT, ksteps, CALL)             \
+  switch (ksteps) {                                        \
+    case 9: CALL(DT, 9); break;                            \
+    case 10: CALL(DT, 10); break;                          \
+    case 11: CALL(DT, 11); break;                          \
+    case 12: CALL(DT, 12); break;                          \
+    case 13: CALL(DT, 13); break;                          \
+    case 14: CALL(DT, 14); break;                          \
+    case 15: CALL(DT, 15); break;                          \
+    default: CALL(DT, 16); break;                          \
   }
 
 #define FCR_DISPATCH_KS4(DT, ksteps, CALL)                 \
@@ -2489,8 +2492,20 @@ void fcr_detail::sweeps_f32(int which, const Params& p, int ksteps, bool causal,
 #endif
 #if FCR_HAS(4)
 void fcr_detail::sweeps_f32_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
-  if (which == 0) { FCR_DISPATCH_KS_F32_LONG(ksteps, FCR_CALL_LSE) }
-  else { FCR_DISPATCH_KS_F32_LONG(ksteps, FCR_CALL_COL) }
+  if (which == 0) { FCR_DISPATCH_KS_LONG(FCR_DTYPE_F32, ksteps, FCR_CALL_LSE) }
+  else { FCR_DISPATCH_KS_LONG(FCR_DTYPE_F32, ksteps, FCR_CALL_COL) }
+}
+#endif
+#if FCR_HAS(5)
+void fcr_detail::sweeps_f16_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
+  if (which == 0) { FCR_DISPATCH_KS_LONG(FCR_DTYPE_F16, ksteps, FCR_CALL_LSE) }
+  else { FCR_DISPATCH_KS_LONG(FCR_DTYPE_F16, ksteps, FCR_CALL_COL) }
+}
+#endif
+#if FCR_HAS(6)
+void fcr_detail::sweeps_bf16_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
+  if (which == 0) { FCR_DISPATCH_KS_LONG(FCR_DTYPE_BF16, ksteps, FCR_CALL_LSE) }
+  else { FCR_DISPATCH_KS_LONG(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL) }
 }
 #endif
 #undef FCR_CALL_LSE
@@ -2505,10 +2520,10 @@ void launch_sweeps(int dtype, int which, const Params& p, int ksteps, bool causa
                    unsigned* zero = nullptr, int zero_words = 0) {
   if (zero_words > 0)
     hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((zero_words + 255) / 256)), dim3(256), 0, s, zero, zero_words);
-  if (dtype == FCR_DTYPE_F16) fcr_detail::sweeps_f16(which, p, ksteps, causal, mode, s);
-  else if (dtype == FCR_DTYPE_BF16) fcr_detail::sweeps_bf16(which, p, ksteps, causal, mode, s);
-  else if (ksteps <= kMaxKSteps) fcr_detail::sweeps_f32(which, p, ksteps, causal, mode, s);
-  else fcr_detail::sweeps_f32_long_rows(which, p, ksteps, causal, mode, s);
+  const bool long_rows = ksteps > kMaxKSteps;
+  if (dtype == FCR_DTYPE_F16) (long_rows ? fcr_detail::sweeps_f16_long_rows : fcr_detail::sweeps_f16)(which, p, ksteps, causal, mode, s);
+  else if (dtype == FCR_DTYPE_BF16) (long_rows ? fcr_detail::sweeps_bf16_long_rows : fcr_detail::sweeps_bf16)(which, p, ksteps, causal, mode, s);
+  else (long_rows ? fcr_detail::sweeps_f32_long_rows : fcr_detail::sweeps_f32)(which, p, ksteps, causal, mode, s);
 }
 
 template <int VPT, typename ET>

@@ -37,8 +37,11 @@ def _validate(query: torch.Tensor, key: torch.Tensor, reduction: Optional[str]):
         )
     if query.device != key.device:
         raise ValueError("Query and key tensors must be on the same device.")
-    if query.shape[3] > 256:
-        raise ValueError(f"Head dimension must be <= 256. Got {query.shape[3]}.")
+    # rows of at most 1 KiB (the reference pads any D to a power of two, flash.py:368-373, and runs what fits
+    # its shared memory)
+    limit = 1024 // query.element_size()
+    if query.shape[3] > limit:
+        raise ValueError(f"Head dimension must be <= {limit} for {query.dtype}. Got {query.shape[3]}.")
 
 
 def _device_layout(x: torch.Tensor) -> torch.Tensor:
@@ -214,7 +217,7 @@ def flash_colreduce(
     """Per-key sum / mean / max over queries of softmax(Q K^T * scale), shape (B, H, N).
 
     Args follow the reference (flash.py:311-352): query (B,H,M,D), key (B,H,N,D), fp16, bf16 or
-    fp32 on the GPU, D <= 256 (fp32 operands are multiplied in fp32); `is_causal` applies the right-aligned mask (key j visible to query i iff
+    fp32 on the GPU, rows of at most 1 KiB: D <= 512, D <= 256 for fp32 (fp32 operands are multiplied in fp32); `is_causal` applies the right-aligned mask (key j visible to query i iff
     j <= i + max(N-M, 0)); `scale` defaults to 1/sqrt(D).
 
     `out_dtype` (keyword only, not in the reference) selects the result dtype.  None reproduces

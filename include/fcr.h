@@ -12,7 +12,7 @@
  *   - q is [B,H,M,D], k is [B,H,N,D], fp16, bf16 or fp32 elements (dtype below).  Strides are in
  *     ELEMENTS, order (batch, head, row, d); the d stride must be 1, row/head/batch strides must be
  *     multiples of 16 bytes (8 16-bit elements, 4 floats) and the base pointers 16-byte aligned; a row
- *     must be a multiple of 16 bytes and D at most 256: D a multiple of 8 in [8, 256] for
+ *     must be a multiple of 16 bytes and at most 1 KiB long: D a multiple of 8 in [8, 512] for
  *     16-bit elements, a multiple of 4 in [4, 256] for fp32.  Rows must not overlap (row stride >= D).
  *     (The reference takes any strides, flash.py:292-299; a caller with other layouts makes a
  *     contiguous, zero-padded copy first -- the Python host does.)  fp32 operands are multiplied at
@@ -58,7 +58,7 @@ extern "C" {
 /* argument errors */
 #define FCR_E_NULL -1      /* a required pointer is NULL */
 #define FCR_E_DTYPE -2     /* dtype is not FCR_DTYPE_* */
-#define FCR_E_SHAPE -3     /* B,H,M,N < 1, D > 256 or a row of D elements not a multiple of 16 bytes, sizes overflow */
+#define FCR_E_SHAPE -3     /* B,H,M,N < 1, a row of D elements longer than 1 KiB or not a multiple of 16 bytes, sizes overflow */
 #define FCR_E_STRIDE -4    /* d stride != 1 or a stride / base pointer breaks 16-byte alignment */
 #define FCR_E_REDUCTION -5 /* reduction is not FCR_REDUCE_* */
 #define FCR_E_SCALE -6     /* scale is not finite */

@@ -70,7 +70,7 @@ def test_c_abi_rejects_bad_arguments_without_a_device(fn):
         (dict(q=None), -1), (dict(k=None), -1), (dict(lse=None), -1), (dict(qs=None), -1),
         (dict(dtype=3), -2), (dict(dtype=-1), -2),
         (dict(B=0), -3), (dict(M=0), -3), (dict(N=-4), -3), (dict(D=0), -3), (dict(D=12), -3),
-        (dict(D=264), -3), (dict(M=(1 << 30) + 1), -3),
+        (dict(D=520), -3), (dict(D=516), -3), (dict(M=(1 << 30) + 1), -3),
         (dict(dtype=2, D=260), -3), (dict(dtype=2, D=6), -3),                 # fp32: a multiple of 4, at most 256
         (dict(dtype=2, D=64, qs=(512, 512, 66, 1)), -4),                       # fp32: strides in multiples of 4
         (dict(qs=(512, 512, 64, 2)), -4), (dict(ks=(512, 512, 60, 1)), -4), (dict(q=18), -4),

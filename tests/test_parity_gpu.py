@@ -204,6 +204,24 @@ def test_head_dims_above_128(m, n, d, causal, dtype):
     run_all(q, k, causal, what=f"m{m} n{n} d{d} {dtype}")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n,d", [(300, 420, 264), (257, 129, 320), (130, 1000, 512), (64, 64, 400),
+                                   (1, 700, 500), (520, 520, 384), (40, 3000, 512), (200, 200, 257), (90, 300, 449)])
+def test_head_dims_above_256(m, n, d, causal, dtype):
+    """D in (256, 512] for 16-bit elements: rows of up to 1 KiB, 9 to 16 k-steps, one workgroup per CU
+    (the reference pads such a D to 512 and runs it when it fits, flash.py:368-373); every k-step count,
+    D that is no multiple of 8 (padded by the host), few queries against many keys (split row sweep)."""
+    q, k = _inputs.randn_pair(1, 3, m, n, d, seed=d + m, dtype=dtype)
+    run_all(q, k, causal, what=f"m{m} n{n} d{d} {dtype}")
+
+
+def test_every_k_step_count_of_long_16_bit_rows():
+    for d in range(264, 513, 32):     # 264, 296, ..: 9 to 16 k-steps of 32 elements
+        q, k = _inputs.randn_pair(2, 2, 150, 333, d, seed=d)
+        run_all(q.half(), k.half(), True, what=f"d{d}")
+
+
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("b,h,m,n,d", [(1, 4, 40, 5000, 64), (1, 32, 128, 4096, 128), (1, 1, 300, 3001, 128),
                                        (2, 3, 1, 2048, 32), (1, 2, 257, 1100, 72)])
@@ -912,6 +930,36 @@ def test_random_shapes_against_oracle():
             check(got, colreduce_ref(q, k, red, causal, scale=scale), red, what)
 
 
+def test_random_decode_shapes_and_fp32_against_oracle():
+    """Second seeded sweep: few queries against many keys (single sweep and its neighbours on either side of
+    its limits: 128 queries, 1024 keys, rows of 256 bytes) and fp32 operands of any shape."""
+    import random
+    rng = random.Random(977)
+    for case in range(60):
+        b, h = rng.randint(1, 2), rng.randint(1, 6)
+        if case % 3 == 2:
+            dtype = torch.float32
+            m = rng.choice([1, 5, 64, 100, 129, 300])
+            n = rng.choice([7, 130, 513, 1500, 2600])
+            d = rng.choice([4, 12, 64, 100, 128, 200, 256])
+        else:
+            dtype = rng.choice([torch.float16, torch.bfloat16])
+            m = rng.choice([1, 2, 16, 33, 63, 64, 65, 100, 127, 128, 129, 140])
+            n = rng.choice([960, 1023, 1024, 1025, 1100, 2047, 2049, 3000, 4097, 7000, 9001])
+            d = rng.choice([8, 32, 64, 72, 128, 136])
+        causal = rng.random() < 0.5
+        scale = rng.choice([None, None, 0.05, 0.4])
+        q, k = _inputs.randn_pair(b, h, m, n, d, seed=5000 + case, dtype=dtype)
+        if rng.random() < 0.3:  # [B, rows, H, D] storage
+            q = q.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+            k = k.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+        reds = rng.sample(REDUCTIONS, rng.randint(1, 3))
+        what = f"case {case}: b{b} h{h} m{m} n{n} d{d} {dtype} causal={causal} scale={scale} {reds}"
+        for red in reds:   # one call per reduction: the calls that may take the single sweep
+            got = fca.flash_colreduce(q.cuda(), k.cuda(), red, is_causal=causal, scale=scale, out_dtype=torch.float32)
+            check(got, colreduce_ref(q, k, red, causal, scale=scale), red, what)
+
+
 def test_hip_graph_capture_and_replay():
     """The whole call (torch allocations, both kernels, cast) captured in a graph and replayed with
     new contents in the static inputs; every replay must equal the eager result for those contents."""
@@ -1016,6 +1064,11 @@ def test_plain_c_caller_of_the_c_abi():
 def test_python_errors_on_device():
     q = torch.zeros(1, 2, 4, 8, dtype=torch.float16, device="cuda")
     k = torch.zeros(1, 2, 6, 8, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError, match="Head dimension must be <= 512"):
+        fca.flash_colreduce(torch.zeros(1, 1, 4, 513, dtype=torch.float16, device="cuda"),
+                            torch.zeros(1, 1, 4, 513, dtype=torch.float16, device="cuda"), "sum")
+    with pytest.raises(ValueError, match="Head dimension must be <= 256"):
+        fca.flash_colreduce(torch.zeros(1, 1, 4, 260, device="cuda"), torch.zeros(1, 1, 4, 260, device="cuda"), "sum")
     with pytest.raises(ValueError, match="Invalid reduction: median"):
         fca.flash_colreduce(q, k, "median")
     with pytest.raises(ValueError, match="same batch size, number of heads, and head dimension"):
