@@ -27,8 +27,9 @@
 // where s_ij = scale * log2(e) * <q_i, k_j>.  The column kernels store the result type of the caller's choice
 // and divide the means as they store (store_column).  The streamed operand goes from global memory straight
 // into a swizzled ring of LDS stages (buffer loads with the LDS as destination).  Nothing of size M*N
-// is written anywhere and there are no atomics on global memory: one workgroup owns its output rows /
-// columns.
+// is written anywhere and nothing in global memory is updated by read-modify-write atomics: one workgroup
+// owns its output rows / columns (col_fused_kernel hands its partial row values to its team with atomic
+// 64-bit stores and loads, value and round number in one word).
 //
 // Replaces the Triton kernel of the reference (flash_colreduce/flash.py:11-274).
 
