@@ -121,10 +121,14 @@ def run_topk(out=sys.stdout):
         b.synchronize()
         return a.elapsed_time(b) / 50 * 1e3
 
-    print(f"{'rows x columns, k':<28} {'topk_keep_mask us':>18} {'torch.topk us':>14} {'topk+scatter us':>16}", file=out)
+    print(f"{'rows x columns, k':<34} {'topk_keep_mask us':>18} {'torch.topk us':>14} {'topk+scatter us':>16}", file=out)
     g = torch.Generator(device="cuda").manual_seed(0)
-    for rows, n, k in TOPK_SHAPES:
-        s = torch.rand(rows, n, device="cuda", generator=g)
+    cases = [(r, n, k, torch.float32) for r, n, k in TOPK_SHAPES]
+    # 16-bit rows, what flash_colreduce returns for 16-bit operands (many ties: the masks may differ in which
+    # of the equal values they keep, so only the number kept and the threshold are compared)
+    cases += [(32, 8192, 2048, torch.float16), (32, 32768, 8192, torch.bfloat16), (32, 262144, 65536, torch.float16)]
+    for rows, n, k, dt in cases:
+        s = torch.rand(rows, n, device="cuda", generator=g).to(dt)
 
         def via_torch():
             idx = torch.topk(s, k, dim=-1).indices
@@ -133,8 +137,13 @@ def run_topk(out=sys.stdout):
         t_ours = timed(lambda: topk_keep_mask(s, k))
         t_topk = timed(lambda: torch.topk(s, k, dim=-1))
         t_mask = timed(via_torch)
-        assert torch.equal(topk_keep_mask(s, k), via_torch())   # distinct values: both masks are the same set
-        print(f"[{rows}, {n}], k={k:<12} {t_ours:>18.1f} {t_topk:>14.1f} {t_mask:>16.1f}", file=out, flush=True)
+        if dt == torch.float32:
+            assert torch.equal(topk_keep_mask(s, k), via_torch())   # distinct values: both masks are the same set
+        else:
+            mask, thr = topk_keep_mask(s, k, return_threshold=True)
+            assert bool((mask.sum(-1) == k).all()) and torch.equal(thr, torch.topk(s, k, dim=-1).values[:, -1].float())
+        label = f"[{rows}, {n}], k={k} {str(dt)[6:]}"
+        print(f"{label:<34} {t_ours:>18.1f} {t_topk:>14.1f} {t_mask:>16.1f}", file=out, flush=True)
 
 
 def main():
