@@ -38,6 +38,7 @@
 #include <stdint.h>
 #include <stdio.h>
 
+#include <mutex>
 #include <type_traits>
 
 #include "fcr.h"
@@ -2741,6 +2742,59 @@ int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, in
 }
 
 namespace {
+// A single sweep expects the whole chip: its workgroups wait for each other, one per CU.  Two of them issued on
+// different streams could be dispatched side by side, each holding CUs the other needs, until their bounded
+// waits run out.  So inside a process they are chained: a single sweep on another stream than the one before
+// first waits (on the GPU; the host never blocks) for an event recorded at the end of that stream.  Calls that
+// stay on one stream pay nothing (an event behind every call costs 5 us of a 18 us call).  Not under stream
+// capture (a graph carries no such edge; graphs holding single sweeps must not replay side by side on one GPU),
+// not for other processes on the same GPU, and not for fcr_colreduce_static, whose calls must not overlap anyway.
+struct SweepOrder {
+  hipEvent_t done = nullptr;
+  hipStream_t last = nullptr;
+  bool any = false;
+};
+SweepOrder g_order[64];
+std::mutex g_order_mu;
+
+// Takes the lock and returns the device's entry when the launch on stream s is to be chained, else nullptr.
+SweepOrder* order_begin(hipStream_t s) {
+  hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(s, &st) != hipSuccess || st != hipStreamCaptureStatusNone) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  g_order_mu.lock();
+  SweepOrder* o = &g_order[dev];
+  if (!o->done && hipEventCreateWithFlags(&o->done, hipEventDisableTiming) != hipSuccess) {
+    (void)hipGetLastError();
+    o->done = nullptr;
+    g_order_mu.unlock();
+    return nullptr;
+  }
+  if (o->any && o->last != s) {
+    // (a stream that is being captured now, or was destroyed, is left alone: nothing of it can still run)
+    hipStreamCaptureStatus lst = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(o->last, &lst) != hipSuccess || lst != hipStreamCaptureStatusNone ||
+        hipEventRecord(o->done, o->last) != hipSuccess || hipStreamWaitEvent(s, o->done, 0) != hipSuccess)
+      (void)hipGetLastError();
+  }
+  return o;
+}
+void order_end(SweepOrder* o, hipStream_t s, bool launched_it) {
+  if (!o) return;
+  if (launched_it) {
+    o->last = s;
+    o->any = true;
+  }
+  g_order_mu.unlock();
+}
+
 // Both sweeps of a call, writing `out` in its final form.  ws_bytes = bytes the caller's workspace is known
 // to have (0: what fcr_lse_bytes asks for).  Few queries against many keys take the single sweep.
 int whole_call(const void* q, const void* k, void* out, const ResultSpec& res, float* ws, size_t ws_bytes, int dtype,
@@ -2771,9 +2825,12 @@ int whole_call(const void* q, const void* k, void* out, const ResultSpec& res, f
     p.stream_once = ((int64_t)p.bh_count * N * p.dgran * 16 >= (1ll << 30)) ? 1 : 0;
     const int words = (int)(f.floats - f.part_at);   // the slots and the error word start at zero
     fcr_detail::fused_refused = false;
+    SweepOrder* const order = (ws_bytes == 0) ? order_begin(s) : nullptr;
     launch_sweeps(dtype, 3, p, ksteps, causal != 0, mode | (f.qh == 2 ? 4 : 0), s, reinterpret_cast<unsigned*>(p.part),
                   words);
-    if (!fcr_detail::fused_refused) return launched("col_fused_kernel");
+    const int lrc = fcr_detail::fused_refused ? 0 : launched("col_fused_kernel");
+    order_end(order, s, !fcr_detail::fused_refused && lrc == 0);
+    if (!fcr_detail::fused_refused) return lrc;
   }
   rc = fcr_row_lse(q, k, ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream);
   if (rc) return rc;

@@ -29,9 +29,10 @@
  *   - Return value: 0 on success; negative FCR_E_* for a rejected argument (nothing was
  *     launched); positive = the hipError_t of a failed launch.  fcr_last_error() returns a
  *     thread-local, human readable description of the last non-zero return on this thread.
- *   - Thread safety: no mutable global state except the thread-local error text and the switches of
- *     fcr_set_option; calls from several threads or streams do not interfere (each call needs its own
- *     lse / workspace buffer while it runs).
+ *   - Thread safety: no mutable global state except the thread-local error text, the switches of
+ *     fcr_set_option and the per-device record of the stream that ran the last single sweep (below); calls
+ *     from several threads or streams do not interfere (each call needs its own lse / workspace buffer
+ *     while it runs).
  */
 #ifndef FCR_H
 #define FCR_H
@@ -206,6 +207,14 @@ int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, in
  * under a CU mask) stores NaN columns for that pair, sets a word in the workspace and goes on.
  * fcr_colreduce_status waits for the stream and returns FCR_E_WAIT if that happened in the last call that
  * used lse_ws with these sizes, 0 otherwise (also for problems that do not take the single sweep).
+ * A single sweep fills the chip, one workgroup per CU, and two of them dispatched side by side would
+ * starve each other until their waits run out.  Inside a process the library prevents that: a single
+ * sweep issued on another stream than the previous one is made to wait on the GPU (an event recorded on
+ * that stream, hipStreamWaitEvent on the new one; the host does not block, calls that stay on one stream
+ * pay nothing).  Outside its reach: launches recorded under stream capture (graphs that hold single
+ * sweeps must not replay side by side on one GPU), other processes on the same GPU, and
+ * fcr_colreduce_static, whose calls must not overlap anyway.  There, switch the single sweep off or
+ * keep such calls apart.
  * No counterpart in the reference, whose kernel has no cross-program dependencies.
  */
 int fcr_colreduce_status(const float* lse_ws, int dtype, int B, int H, int M, int N, int D, void* stream);

@@ -459,6 +459,29 @@ def test_single_sweep_bounded_wait():
     assert lib.fcr_set_option(7, 1) == -3 and lib.fcr_set_option(_lib.OPT_WAIT_POLLS, -1) == -3
 
 
+def test_single_sweeps_on_two_streams_are_chained():
+    """A single sweep expects the whole chip (its workgroups wait for each other), so the library chains the
+    single sweeps that a process issues on different streams with an event: calls issued alternately on two
+    streams, with no host synchronisation between them, all give the results of the calls made alone."""
+    qa, ka = _inputs.randn_pair(2, 8, 64, 8192, 128, seed=5, dtype=torch.float16)
+    qb, kb = _inputs.randn_pair(1, 16, 128, 4096, 64, seed=6, dtype=torch.bfloat16)
+    qa, ka, qb, kb = qa.cuda(), ka.cuda(), qb.cuda(), kb.cuda()
+    want_a = fca.flash_colreduce(qa, ka, "sum", is_causal=True)
+    want_b = fca.flash_colreduce(qb, kb, "max", is_causal=False)
+    check(want_a.float().cpu(), colreduce_ref(qa.cpu(), ka.cpu(), "sum", True), "sum", "alone")
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    got = []
+    for _ in range(25):
+        with torch.cuda.stream(sa):
+            got.append((want_a, fca.flash_colreduce(qa, ka, "sum", is_causal=True)))
+        with torch.cuda.stream(sb):
+            got.append((want_b, fca.flash_colreduce(qb, kb, "max", is_causal=False)))
+    torch.cuda.synchronize()
+    for want, out in got:
+        assert torch.equal(out, want)
+
+
 def test_single_sweep_under_graph_capture():
     """The single sweep (a small kernel that clears the slots, then the sweep) captured and replayed."""
     b, h, m, n, d = 2, 8, 64, 4096, 128
