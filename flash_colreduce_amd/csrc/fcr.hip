@@ -1192,7 +1192,9 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
   constexpr int kRes = (MODE == kModeBoth) ? 2 : 1;
   constexpr int kObufFloats = QH * kRes * kItemKeys;
   constexpr int kRedFloats = 8 * 64;
-  constexpr int kMergeWaves = 8 / QH;            // waves per row that share the merge of the team's partial values
+  // waves per row that share the merge of the team's partial values (half of them when two results are
+  // buffered for 1024 keys: the LDS is full)
+  constexpr int kMergeWaves = (8 / QH) / ((kRes == 2 && QH == 1) ? 2 : 1);
   constexpr int kBatch = 4 * QH;                 // slots a lane fetches together: one round trip for teams of up to 32
   constexpr int kMrgFloats = kMergeWaves * kRowsWg * 2;
   constexpr int kAhead = NS / KH - 1;            // steps in flight in front of the one being computed
@@ -1522,7 +1524,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     // All waves share the team's slots: lane = row, the waves of a row take every kMergeWaves-th slot, poll
     // until it carries this round, and fold the values into (max, sum).  (The keys a wave has in flight
     // for the next pair return before these loads do; they were requested during the last steps above.)
-    {
+    if (wave / QH < kMergeWaves) {
       const int rgroup = wave % QH, sub = wave / QH;
       const unsigned long long* mine = slots + 64 * rgroup + lane;
       float m = kNegInf, acc = 0.f;
@@ -2413,16 +2415,18 @@ void launch_col_fused_mode(const Params& p, bool causal, hipStream_t s) {
   else hipLaunchKernelGGL((col_fused_kernel<DT, KS, false, MODE, QH>), grid, block, 0, s, p);
 }
 
-// mode: kModeSum or kModeMax, + 4 for more than 64 queries
+// mode: kModeSum, kModeMax or kModeBoth, + 4 for more than 64 queries
 template <int DT, int KS>
 void launch_col_fused(const Params& p, bool causal, int mode, hipStream_t s) {
   const int m = mode & 3;
   if (mode & 4) {
     if (m == kModeSum) launch_col_fused_mode<DT, KS, kModeSum, 2>(p, causal, s);
-    else launch_col_fused_mode<DT, KS, kModeMax, 2>(p, causal, s);
+    else if (m == kModeMax) launch_col_fused_mode<DT, KS, kModeMax, 2>(p, causal, s);
+    else launch_col_fused_mode<DT, KS, kModeBoth, 2>(p, causal, s);
   } else {
     if (m == kModeSum) launch_col_fused_mode<DT, KS, kModeSum, 1>(p, causal, s);
-    else launch_col_fused_mode<DT, KS, kModeMax, 1>(p, causal, s);
+    else if (m == kModeMax) launch_col_fused_mode<DT, KS, kModeMax, 1>(p, causal, s);
+    else launch_col_fused_mode<DT, KS, kModeBoth, 1>(p, causal, s);
   }
 }
 
@@ -2799,7 +2803,7 @@ void order_end(SweepOrder* o, hipStream_t s, bool launched_it) {
 // to have (0: what fcr_lse_bytes asks for).  Few queries against many keys take the single sweep.
 int whole_call(const void* q, const void* k, void* out, const ResultSpec& res, float* ws, size_t ws_bytes, int dtype,
                int B, int H, int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
-               int mode, int causal, void* stream) {
+               int mode, int causal, void* stream, void* out2 = nullptr) {
   Params p;
   int rc = make_params(p, q, k, dtype, B, H, M, N, D, q_strides, k_strides, scale, true, causal != 0, mode);
   if (rc) return rc;
@@ -2817,6 +2821,7 @@ int whole_call(const void* q, const void* k, void* out, const ResultSpec& res, f
     const long long polls = __atomic_load_n(&g_wait_polls, __ATOMIC_RELAXED);
     p.spin_limit = polls > 0x7fffffffll ? 0x7fffffff : (int)polls;
     p.out = out;
+    p.out2 = out2;
     p.out_fmt = res.fmt;
     if (res.mean) {
       p.mean_from = causal ? p.c : N;
@@ -2834,10 +2839,18 @@ int whole_call(const void* q, const void* k, void* out, const ResultSpec& res, f
   }
   rc = fcr_row_lse(q, k, ws, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream);
   if (rc) return rc;
-  return col_reduce_any(q, k, ws, out, nullptr, mode, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream,
+  return col_reduce_any(q, k, ws, out, out2, mode, dtype, B, H, M, N, D, q_strides, k_strides, scale, causal, stream,
                         res);
 }
 }  // namespace
+
+int fcr_colreduce_sum_max(const void* q, const void* k, float* out_sum, float* out_max, float* lse_ws, int dtype, int B,
+                          int H, int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
+                          float scale, int causal, void* stream) {
+  if (!out_sum || !out_max || !lse_ws) return fail(FCR_E_NULL, "null pointer argument");
+  return whole_call(q, k, out_sum, ResultSpec(), lse_ws, 0, dtype, B, H, M, N, D, q_strides, k_strides, scale, kModeBoth,
+                    causal, stream, out_max);
+}
 
 int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H, int M,
                   int N, int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,

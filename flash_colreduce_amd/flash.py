@@ -164,12 +164,10 @@ def _launch(query, key, kinds, is_causal, scale):
                 _lib.check(lib.fcr_colreduce(q.data_ptr(), k.data_ptr(), outs[0].data_ptr(), lse.data_ptr(),
                                              *common, red, causal, stream))
             elif sorted(kinds) == ["max", "sum"]:
-                # both kinds from one column sweep
+                # both kinds from one column sweep (few queries against many keys: from the single sweep)
                 by_kind = dict(zip(kinds, outs))
-                _lib.check(lib.fcr_row_lse(q.data_ptr(), k.data_ptr(), lse.data_ptr(), *common, causal, stream))
-                _lib.check(lib.fcr_col_reduce_sum_max(q.data_ptr(), k.data_ptr(), lse.data_ptr(),
-                                                      by_kind["sum"].data_ptr(), by_kind["max"].data_ptr(),
-                                                      *common, causal, stream))
+                _lib.check(lib.fcr_colreduce_sum_max(q.data_ptr(), k.data_ptr(), by_kind["sum"].data_ptr(),
+                                                     by_kind["max"].data_ptr(), lse.data_ptr(), *common, causal, stream))
             else:
                 _lib.check(lib.fcr_row_lse(q.data_ptr(), k.data_ptr(), lse.data_ptr(), *common, causal, stream))
                 for kind, o in zip(kinds, outs):

@@ -44,7 +44,7 @@
 extern "C" {
 #endif
 
-#define FCR_VERSION 310 /* major*10000 + minor*100 + patch */
+#define FCR_VERSION 320 /* major*10000 + minor*100 + patch */
 
 /* element type of q and k */
 #define FCR_DTYPE_F16 0
@@ -166,6 +166,15 @@ int fcr_pack_f32(const float* src, void* dst, int64_t rows, int D, int terms, in
 int fcr_colreduce(const void* q, const void* k, float* out, float* lse_ws, int dtype, int B, int H,
                   int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
                   float scale, int reduction, int causal, void* stream);
+
+/*
+ * fcr_colreduce for the column sums AND the column maxima of one problem (the reference makes two full calls,
+ * flash.py:311-385 once per reduction): one row pass and one column sweep, or, for few queries against many
+ * keys, one single sweep.  out_sum and out_max are fp32 [B*H, N]; lse_ws as for fcr_colreduce.
+ */
+int fcr_colreduce_sum_max(const void* q, const void* k, float* out_sum, float* out_max, float* lse_ws, int dtype, int B,
+                          int H, int M, int N, int D, const int64_t q_strides[4], const int64_t k_strides[4],
+                          float scale, int causal, void* stream);
 
 /*
  * The whole operator as the reference's caller sees it: both kernels, the cast of the fp32 accumulation

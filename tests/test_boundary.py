@@ -28,14 +28,14 @@ def test_library_exports_every_declared_symbol():
     assert {"fcr_version", "fcr_last_error", "fcr_lse_bytes", "fcr_row_lse", "fcr_col_reduce",
             "fcr_col_reduce_sum_max", "fcr_pack_f32", "fcr_colreduce", "fcr_colreduce_static",
             "fcr_colreduce_to", "fcr_topk_mask", "fcr_topk_mask_ws", "fcr_topk_mask_typed", "fcr_topk_bytes", "fcr_set_option",
-            "fcr_colreduce_status"} <= set(names)
+            "fcr_colreduce_status", "fcr_colreduce_sum_max"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
 
 
 def test_version_and_sizes():
     lib = _lib.load()
-    assert lib.fcr_version() == 310
+    assert lib.fcr_version() == 320
     assert lib.fcr_lse_bytes(2, 3, 5, 7, 64) == 2 * 3 * 5 * 4
     assert lib.fcr_lse_bytes(1, 32, 8192, 8192, 128) == 32 * 8192 * 4      # enough row tiles: no scratch
     assert lib.fcr_lse_bytes(1, 32, 512, 16384, 128) == 32 * 512 * 4 * 9   # 8 key ranges + the result
@@ -59,10 +59,13 @@ def _call(lib, fn, **over):
     if fn == "colreduce_to":
         return lib.fcr_colreduce_to(a["q"], a["k"], a["out"], a.get("out_dtype", 0), a["lse"], *common, a["red"],
                                     a["causal"], None)
+    if fn == "colreduce_sum_max":
+        return lib.fcr_colreduce_sum_max(a["q"], a["k"], a["out"], a.get("out_max", 80), a["lse"], *common, a["causal"],
+                                         None)
     return lib.fcr_colreduce(a["q"], a["k"], a["out"], a["lse"], *common, a["red"], a["causal"], None)
 
 
-@pytest.mark.parametrize("fn", ["row_lse", "col_reduce", "colreduce", "colreduce_to"])
+@pytest.mark.parametrize("fn", ["row_lse", "col_reduce", "colreduce", "colreduce_to", "colreduce_sum_max"])
 def test_c_abi_rejects_bad_arguments_without_a_device(fn):
     """Every rejection happens before the first HIP call, so fake pointers are safe here."""
     lib = _lib.load()
@@ -83,6 +86,8 @@ def test_c_abi_rejects_bad_arguments_without_a_device(fn):
     if fn == "colreduce_to":   # takes the mean as a third reduction, and a result type
         cases += [(dict(out=None), -1), (dict(red=3), -5), (dict(red=-1), -5), (dict(out_dtype=3), -2),
                   (dict(out_dtype=-1), -2)]
+    elif fn == "colreduce_sum_max":
+        cases += [(dict(out=None), -1), (dict(out_max=None), -1)]
     elif fn != "row_lse":
         cases += [(dict(out=None), -1), (dict(red=2), -5), (dict(red=-1), -5)]
     for over, code in cases:

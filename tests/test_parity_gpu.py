@@ -381,6 +381,13 @@ def test_single_sweep(b, h, m, n, d, causal, dtype):
     torch.testing.assert_close(got, two, rtol=2e-5, atol=1e-7)
     torch.testing.assert_close(lse, lse2, rtol=0, atol=2e-5)
     assert torch.equal(got, _c_abi_colreduce(qd, kd, "sum", causal)[0])   # no atomic adds: repeatable bit for bit
+    # sums and maxima from the same single sweep (fcr_colreduce_sum_max)
+    both_sum, both_max = fca.flash_colreduce_multi(qd, kd, ["sum", "max"], is_causal=causal, out_dtype=torch.float32)
+    check(both_sum.cpu(), colreduce_ref(q, k, "sum", causal), "sum", what + " both")
+    check(both_max.cpu(), colreduce_ref(q, k, "max", causal), "max", what + " both")
+    torch.testing.assert_close(both_sum, got, rtol=2e-5, atol=1e-7)
+    # (the team's partial values are merged by half as many waves, in another order: equal to rounding)
+    torch.testing.assert_close(both_max.view(b, h, n), _c_abi_colreduce(qd, kd, "max", causal)[0], rtol=2e-5, atol=0)
 
 
 @pytest.mark.parametrize("causal", [False, True])
