@@ -48,6 +48,9 @@ def _declare(lib):
                                    [c.c_int, c.c_int, c.c_void_p])
     lib.fcr_colreduce_sum_max.restype = c.c_int
     lib.fcr_colreduce_sum_max.argtypes = ([c.c_void_p] * 5 + common + [c.c_int, c.c_void_p])
+    lib.fcr_colreduce_sum_max_to.restype = c.c_int
+    lib.fcr_colreduce_sum_max_to.argtypes = ([c.c_void_p] * 4 + [c.c_int, c.c_void_p] + common +
+                                             [c.c_int, c.c_int, c.c_void_p])
     lib.fcr_col_reduce_sum_max.restype = c.c_int
     lib.fcr_col_reduce_sum_max.argtypes = ([c.c_void_p] * 5 + common + [c.c_int, c.c_void_p])
     lib.fcr_topk_mask.restype = c.c_int

@@ -2907,6 +2907,21 @@ int fcr_colreduce_to(const void* q, const void* k, void* out, int out_dtype, flo
                     reduction == FCR_REDUCE_MAX ? kModeMax : kModeSum, causal, stream);
 }
 
+int fcr_colreduce_sum_max_to(const void* q, const void* k, void* out_sum, void* out_max, int out_dtype, float* lse_ws,
+                             int dtype, int B, int H, int M, int N, int D, const int64_t q_strides[4],
+                             const int64_t k_strides[4], float scale, int sum_reduction, int causal, void* stream) {
+  if (!out_sum || !out_max || !lse_ws) return fail(FCR_E_NULL, "null pointer argument");
+  if (sum_reduction != FCR_REDUCE_SUM && sum_reduction != FCR_REDUCE_MEAN)
+    return fail(FCR_E_REDUCTION, "sum_reduction must be FCR_REDUCE_SUM or FCR_REDUCE_MEAN");
+  if (out_dtype != FCR_DTYPE_F16 && out_dtype != FCR_DTYPE_BF16 && out_dtype != FCR_DTYPE_F32)
+    return fail(FCR_E_DTYPE, "out_dtype must be FCR_DTYPE_F16, FCR_DTYPE_BF16 or FCR_DTYPE_F32");
+  ResultSpec res;
+  res.fmt = out_dtype;
+  res.mean = sum_reduction == FCR_REDUCE_MEAN;
+  return whole_call(q, k, out_sum, res, lse_ws, 0, dtype, B, H, M, N, D, q_strides, k_strides, scale, kModeBoth, causal,
+                    stream, out_max);
+}
+
 int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, int B, int H, int M, int N, int D,
                          const int64_t q_strides[4], const int64_t k_strides[4], float scale, int reduction,
                          int causal, void* stream) {

@@ -133,6 +133,27 @@ def _launch_to(query, key, reduction, is_causal, scale, res_dtype):
     return out
 
 
+def _launch_pair_to(query, key, sum_reduction, is_causal, scale, res_dtype):
+    """Sums (or means) and maxima from one call, finished on the device (fcr_colreduce_sum_max_to)."""
+    b, h, m, d = query.shape
+    n = key.shape[2]
+    if scale is None:
+        scale = 1 / math.sqrt(d)  # the unpadded D (flash.py:366-367)
+    q, k = _operands(query, key)
+    lib = _lib.load()
+    dev = query.device
+    index = dev.index if dev.index is not None else torch.cuda.current_device()
+    lse = torch.empty(_lse_floats(index, b, h, m, n, q.shape[3]), device=dev, dtype=torch.float32)
+    sums = torch.empty((b, h, n), device=dev, dtype=res_dtype)
+    maxs = torch.empty((b, h, n), device=dev, dtype=res_dtype)
+    with torch.cuda.device(index):
+        _lib.check(lib.fcr_colreduce_sum_max_to(
+            q.data_ptr(), k.data_ptr(), sums.data_ptr(), maxs.data_ptr(), _DTYPES[res_dtype], lse.data_ptr(),
+            _DTYPES[q.dtype], b, h, m, n, q.shape[3], _lib.strides4(q.stride()), _lib.strides4(k.stride()), float(scale),
+            _REDUCTIONS[sum_reduction], 1 if is_causal else 0, _raw_stream(dev)))
+    return sums, maxs
+
+
 def _launch(query, key, kinds, is_causal, scale):
     """Runs the row kernel once and the column kernel for the entries of `kinds` ('sum' / 'max').
 
@@ -266,6 +287,16 @@ def flash_colreduce_multi(
     res_dtype = query.dtype if out_dtype is None else out_dtype
     if m == 0 and n > 0 and b * h > 0 and "max" in reductions:
         raise ValueError("reduction='max' needs at least one query row.")
+    wanted = set(reductions)
+    if m > 0 and b * h * n > 0 and res_dtype in _DTYPES and wanted in ({"sum", "max"}, {"mean", "max"}):
+        # the usual pair: both results leave the kernel in their final form (fcr_colreduce_sum_max_to)
+        sums, maxs = _launch_pair_to(query, key, "mean" if "mean" in wanted else "sum", is_causal, scale, res_dtype)
+        out, seen = [], set()
+        for r in reductions:   # an entry named twice gets a tensor of its own
+            t = maxs if r == "max" else sums
+            out.append(t.clone() if r in seen else t)
+            seen.add(r)
+        return tuple(out)
     kinds = []
     for r in reductions:
         kind = "max" if r == "max" else "sum"

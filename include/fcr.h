@@ -203,6 +203,16 @@ int fcr_colreduce_to(const void* q, const void* k, void* out, int out_dtype, flo
  * a device asks the runtime for the buffer's address and should be made outside graph capture.
  * Results are bitwise those of fcr_colreduce.
  */
+/*
+ * fcr_colreduce_sum_max with the tail of the reference's wrapper, as fcr_colreduce_to has it: both results
+ * leave the kernel as [B*H, N] of out_dtype, and with sum_reduction = FCR_REDUCE_MEAN (else FCR_REDUCE_SUM)
+ * the sums are divided as in flash.py:377-384.  Stands for two calls of flash_colreduce, 'sum' or 'mean' and
+ * 'max' (flash.py:311-385), bit for bit what those give up to the order of the fp32 additions.
+ */
+int fcr_colreduce_sum_max_to(const void* q, const void* k, void* out_sum, void* out_max, int out_dtype, float* lse_ws,
+                             int dtype, int B, int H, int M, int N, int D, const int64_t q_strides[4],
+                             const int64_t k_strides[4], float scale, int sum_reduction, int causal, void* stream);
+
 int fcr_colreduce_static(const void* q, const void* k, float* out, int dtype, int B, int H, int M, int N,
                          int D, const int64_t q_strides[4], const int64_t k_strides[4], float scale,
                          int reduction, int causal, void* stream);

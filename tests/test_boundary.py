@@ -28,7 +28,7 @@ def test_library_exports_every_declared_symbol():
     assert {"fcr_version", "fcr_last_error", "fcr_lse_bytes", "fcr_row_lse", "fcr_col_reduce",
             "fcr_col_reduce_sum_max", "fcr_pack_f32", "fcr_colreduce", "fcr_colreduce_static",
             "fcr_colreduce_to", "fcr_topk_mask", "fcr_topk_mask_ws", "fcr_topk_mask_typed", "fcr_topk_bytes", "fcr_set_option",
-            "fcr_colreduce_status", "fcr_colreduce_sum_max"} <= set(names)
+            "fcr_colreduce_status", "fcr_colreduce_sum_max", "fcr_colreduce_sum_max_to"} <= set(names)
     for name in names:
         assert hasattr(lib, name), name
 

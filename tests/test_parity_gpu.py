@@ -800,6 +800,37 @@ def test_multi_reduction_shares_the_row_pass(causal):
         fca.flash_colreduce_multi(qd, kd, [])
 
 
+@pytest.mark.parametrize("res_dtype", [None, torch.float32])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m,n,d,dtype", [(300, 5000, 64, torch.bfloat16), (64, 4096, 128, torch.float16),
+                                         (100, 2000, 32, torch.bfloat16), (700, 300, 128, torch.float16)])
+def test_sum_or_mean_with_max_finished_in_the_kernel(m, n, d, dtype, causal, res_dtype):
+    """'sum' or 'mean' together with 'max' is one call of fcr_colreduce_sum_max_to (two kernels, or the single
+    sweep): both results leave it in the result type, the means divided as flash.py:377-384 does.  Held to
+    the torch sequence on the same call's fp32 sums bit for bit, and to the one-reduction calls."""
+    q, k = _inputs.randn_pair(2, 3, m, n, d, seed=m + n, dtype=dtype)
+    qd, kd = q.cuda(), k.cuda()
+    rt = dtype if res_dtype is None else res_dtype
+    s32, x32 = fca.flash_colreduce_multi(qd, kd, ["sum", "max"], is_causal=causal, out_dtype=torch.float32)
+    check(s32.cpu(), colreduce_ref(q, k, "sum", causal), "sum", "pair")
+    check(x32.cpu(), colreduce_ref(q, k, "max", causal), "max", "pair")
+    for red in ("sum", "mean"):
+        got, mx = fca.flash_colreduce_multi(qd, kd, [red, "max"], is_causal=causal, out_dtype=res_dtype)
+        assert got.dtype == rt and mx.dtype == rt and got.shape == (2, 3, n) and mx.shape == (2, 3, n)
+        want = s32.to(rt)
+        if red == "mean":
+            c = max(n - m, 0) if causal else n
+            want[..., :c] /= m
+            if c < n:
+                want[..., c:] /= torch.arange(n - c, 0, -1, device="cuda")
+        assert torch.equal(got, want), red
+        assert torch.equal(mx, x32.to(rt))
+        one = fca.flash_colreduce(qd, kd, red, is_causal=causal, out_dtype=res_dtype)
+        torch.testing.assert_close(got.float(), one.float(), rtol=2e-5 if rt == torch.float32 else 1e-2, atol=1e-7)
+    twice = fca.flash_colreduce_multi(qd, kd, ["max", "mean", "max"], is_causal=causal)
+    assert torch.equal(twice[0], twice[2]) and twice[0].data_ptr() != twice[2].data_ptr()
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("m,n,d", [(1, 1, 8), (131, 1027, 72), (700, 300, 128), (40, 1000, 24), (300, 420, 200),
