@@ -54,7 +54,7 @@ extern "C" {
 /* column reduction over query rows */
 #define FCR_REDUCE_SUM 0 /* also the numerator of 'mean' (flash.py:121-122) */
 #define FCR_REDUCE_MAX 1 /* flash.py:123-124 */
-#define FCR_REDUCE_MEAN 2 /* fcr_colreduce_to only: the sums divided as in flash.py:377-384 */
+#define FCR_REDUCE_MEAN 2 /* fcr_colreduce_to and fcr_colreduce_sum_max_to only: the sums divided as in flash.py:377-384 */
 
 /* argument errors */
 #define FCR_E_NULL -1      /* a required pointer is NULL */

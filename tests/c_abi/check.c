@@ -22,6 +22,17 @@
     }                                                                       \
   } while (0)
 
+/* the closed form of column j */
+static double closed_form(int red, int causal, int M, int N, int j) {
+  const int c = N > M ? N - M : 0;
+  if (!causal) return red == FCR_REDUCE_SUM ? (double)M / N : 1.0 / N;
+  const int first = j > c ? j : c;   /* the first row that sees key j is row first - c, with first + 1 keys */
+  if (red != FCR_REDUCE_SUM) return 1.0 / (first + 1);
+  double want = 0.0;
+  for (int n = first + 1; n <= (M <= N ? N : M + c); ++n) want += (n <= N) ? 1.0 / n : 1.0 / N;
+  return want;
+}
+
 static int run_case(int B, int H, int M, int N, int D, int causal) {
   const size_t qn = (size_t)B * H * M * D, kn = (size_t)B * H * N * D, on = (size_t)B * H * N;
   uint16_t* hk = (uint16_t*)malloc(kn * 2);
@@ -36,7 +47,6 @@ static int run_case(int B, int H, int M, int N, int D, int causal) {
   CHECK_HIP(hipMemset(q, 0, qn * 2));
   CHECK_HIP(hipMemcpy(k, hk, kn * 2, hipMemcpyHostToDevice));
   const int64_t qs[4] = {(int64_t)H * M * D, (int64_t)M * D, D, 1}, ks[4] = {(int64_t)H * N * D, (int64_t)N * D, D, 1};
-  const int c = N > M ? N - M : 0;
   int bad = 0;
   for (int red = FCR_REDUCE_SUM; red <= FCR_REDUCE_MAX; ++red) {
     const int rc = fcr_colreduce(q, k, out, lse, FCR_DTYPE_F16, B, H, M, N, D, qs, ks, 0.125f, red, causal, NULL);
@@ -47,18 +57,7 @@ static int run_case(int B, int H, int M, int N, int D, int causal) {
     CHECK_HIP(hipDeviceSynchronize());
     CHECK_HIP(hipMemcpy(ho, out, on * 4, hipMemcpyDeviceToHost));
     for (int j = 0; j < N; ++j) {
-      double want;
-      if (!causal) {
-        want = red == FCR_REDUCE_SUM ? (double)M / N : 1.0 / N;
-      } else {
-        const int first = j > c ? j : c;   /* the first row that sees key j is row first - c, with first + 1 keys */
-        want = 0.0;
-        if (red == FCR_REDUCE_SUM) {
-          for (int n = first + 1; n <= (M <= N ? N : M + c); ++n) want += (n <= N) ? 1.0 / n : 1.0 / N;
-        } else {
-          want = 1.0 / (first + 1);
-        }
-      }
+      const double want = closed_form(red, causal, M, N, j);
       for (int bh = 0; bh < B * H; ++bh) {
         const double got = ho[(size_t)bh * N + j];
         if (!(fabs(got - want) <= 2e-5 * want)) {
@@ -66,6 +65,31 @@ static int run_case(int B, int H, int M, int N, int D, int causal) {
         }
       }
     }
+  }
+  /* sums and maxima from one call, and the word that says whether every workgroup of a single sweep met its team */
+  {
+    float* out2;
+    CHECK_HIP(hipMalloc((void**)&out2, on * 4));
+    const int rc = fcr_colreduce_sum_max(q, k, out, out2, lse, FCR_DTYPE_F16, B, H, M, N, D, qs, ks, 0.125f, causal, NULL);
+    if (rc != 0) {
+      fprintf(stderr, "fcr_colreduce_sum_max: %d %s\n", rc, fcr_last_error());
+      return 3;
+    }
+    const int st = fcr_colreduce_status(lse, FCR_DTYPE_F16, B, H, M, N, D, NULL);
+    if (st != 0) {
+      fprintf(stderr, "fcr_colreduce_status: %d %s\n", st, fcr_last_error());
+      return 3;
+    }
+    for (int red = FCR_REDUCE_SUM; red <= FCR_REDUCE_MAX; ++red) {
+      CHECK_HIP(hipMemcpy(ho, red == FCR_REDUCE_SUM ? out : out2, on * 4, hipMemcpyDeviceToHost));
+      for (int j = 0; j < N; j += (N > 7 ? N / 7 : 1)) {
+        const double want = closed_form(red, causal, M, N, j), got = ho[(size_t)(B * H - 1) * N + j];
+        if (!(fabs(got - want) <= 2e-5 * want)) {
+          if (bad++ < 5) fprintf(stderr, "sum_max B%d H%d M%d N%d causal%d red%d j%d: got %.9g want %.9g\n", B, H, M, N, causal, red, j, got, want);
+        }
+      }
+    }
+    CHECK_HIP(hipFree(out2));
   }
   CHECK_HIP(hipFree(q));
   CHECK_HIP(hipFree(k));
