@@ -25,6 +25,9 @@ configs      the five named workloads of the benchmark set: ms per call (events,
              back between two events: the time of the call's kernels on the GPU as long as the host issues a
              call faster than that (`host_issue_us`); `ms` is the Python operator, torch allocations included.
              `--configs 2,3` restricts the set (and `--no-headline` skips the headline) for profiler runs.
+decode       the HBM-bound shape of the reference's own benchmark table (causal B=64 H=32 M=64 N=16384 D=128
+             fp16, sum; benchmarks/run.py:34-55): ms per call, and a `roofline` object of its own, the
+             algorithmic bytes over the time of the call's kernels against the 8 TB/s HBM peak.
 """
 from __future__ import annotations
 
@@ -45,6 +48,9 @@ PEAK_HBM_TBPS = 8.0
 # to move (q, k, the fp32 result) that is 1.70 times the bytes for the row sweep and 1.48 for the column
 # sweep: streamed tiles that several workgroups ask for and that do not all meet in a cache.
 HBM_TRAFFIC_BYTES = {"row_lse_kernel": 229.5e6 + 1.05e6, "col_reduce_kernel": 199.7e6 + 1.05e6}
+# the same for the single sweep on the decode workload (profiles/decode_b64_m64_n16384_fp16.md): 9.00 GB read
+# (1.045 times the keys and queries), 84.4 MB written
+DECODE_TRAFFIC_BYTES = 9.00e9 + 84.4e6
 CONDITIONING_SECONDS = 0.4
 CONFIG_CONDITIONING_SECONDS = 0.25   # per workload and reduction of the configs array, untimed
 
@@ -99,6 +105,38 @@ def _c_abi_us(torch, qd, kd, red, causal, reps):
     e1.record()
     e1.synchronize()
     return e0.elapsed_time(e1) / reps * 1e3, host
+
+
+def run_decode(torch, fca, colreduce_ref):
+    """The HBM-bound shape of the reference's benchmark table (benchmarks/run.py:34-55): causal B=64 H=32 M=64
+    N=16384 D=128 fp16, sum.  The single sweep reads the 8.6 GB of keys once; its roofline is the HBM peak.
+    Timed with events through the Python operator and through the C ABI; parity on two (b,h) pairs."""
+    dev = torch.device("cuda:0")
+    b, h, m, n, d = 64, 32, 64, 16384, 128
+    g = torch.Generator(device="cuda").manual_seed(13)
+    qd = torch.randn(b, h, m, d, device=dev, dtype=torch.float16, generator=g)
+    kd = torch.randn(b, h, n, d, device=dev, dtype=torch.float16, generator=g)
+    fn = lambda: fca.flash_colreduce(qd, kd, "sum", is_causal=True, out_dtype=torch.float32)
+    got = fn()
+    for _ in range(5):
+        fn()
+    torch.cuda.synchronize()
+    ms = _events_ms(torch, fn, 20)
+    kernel_us, host_us = _c_abi_us(torch, qd, kd, "sum", True, 20)
+    pick = [(0, 0), (63, 31)]
+    qs = torch.stack([qd[i, j] for i, j in pick]).unsqueeze(0).float().cpu()
+    ks = torch.stack([kd[i, j] for i, j in pick]).unsqueeze(0).float().cpu()
+    want = colreduce_ref(qs, ks, "sum", True)
+    ok, worst = _close(torch, torch.stack([got[i, j] for i, j in pick]).unsqueeze(0).cpu(), want, "sum")
+    bytes_alg = b * h * (m + n) * d * 2 + b * h * n * 4
+    return {"name": "decode_b64_m64_n16384", "shape": {"B": b, "H": h, "M": m, "N": n, "D": d}, "dtype": "float16",
+            "causal": True, "reduction": "sum", "algorithmic_bytes": bytes_alg, "ms": ms, "kernel_us": kernel_us,
+            "host_issue_us": host_us, "launches_per_call": 2,
+            "roofline": {"bound": "hbm", "kernel": "col_fused_kernel", "achieved": bytes_alg / (kernel_us * 1e-6) / 1e9,
+                         "peak": PEAK_HBM_TBPS * 1e3, "unit": "GB/s",
+                         "frac": bytes_alg / (kernel_us * 1e-6) / 1e12 / PEAK_HBM_TBPS,
+                         "traffic": DECODE_TRAFFIC_BYTES},
+            "pass": ok, "worst_err_over_tol": worst}
 
 
 def run_configs(torch, fca, colreduce_ref, inputs, cores, only=None):
@@ -318,6 +356,7 @@ def main():
     torch.cuda.empty_cache()
 
     configs = None if args.no_configs else run_configs(torch, fca, colreduce_ref, _inputs, cores, only)
+    decode = None if args.no_configs else run_decode(torch, fca, colreduce_ref)
 
     line = {
         "metric": METRIC,
@@ -331,6 +370,7 @@ def main():
                    "conditioning": f"{cond_calls} untimed calls of the same workload over {args.conditioning} s "
                                    "before the warm-up (GPU clocks leave idle); not part of warmup or steps"},
         "roofline": roofline, "cpu_baseline": cpu_baseline, "parity": parity, "configs": configs,
+        "decode": decode,
     }
     print(json.dumps(line), flush=True)
 
