@@ -18,7 +18,7 @@ INCLUDE = os.path.join(ROOT, "include")
 LIB = os.path.join(HERE, "libfcr.so")
 
 OBJ_DIR = os.path.join(HERE, "_build")
-PARTS = (0, 1, 2, 3, 4, 5, 6)   # -DFCR_PART=n, see the top of csrc/fcr.hip
+PARTS = (0, 1, 2, 3, 4, 5, 6, 7, 8)   # -DFCR_PART=n, see the top of csrc/fcr.hip
 
 HIPCC_FLAGS = [
     "-O3",

@@ -46,7 +46,7 @@
 // The file can be compiled whole, or in parts that are linked together (the build script does that to
 // use several cores): part 0 holds the C ABI and the small kernels, parts 1-4 the sweeps of one element
 // type each (fp16, bf16, fp32 rows up to 512 bytes, longer fp32 rows), parts 5 and 6 the sweeps over fp16 and
-// bf16 rows of more than 512 bytes.
+// bf16 rows of more than 512 bytes, parts 7 and 8 the single sweep for fp16 and bf16.
 #ifndef FCR_PART
 #define FCR_PART -1
 #endif
@@ -87,6 +87,8 @@ void sweeps_f16(int which, const Params& p, int ksteps, bool causal, int mode, h
 void sweeps_bf16(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_f32(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_f32_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
+void sweeps_f16_single(const Params& p, int ksteps, bool causal, int mode, hipStream_t s);    // col_fused_kernel
+void sweeps_bf16_single(const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_f16_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 void sweeps_bf16_long_rows(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s);
 extern thread_local bool fused_refused;   // set by a launcher of col_fused_kernel that did not launch
@@ -1140,8 +1142,9 @@ __global__ __launch_bounds__(kThreads, (NG <= 4 ? 3 : 2)) void col_small_kernel(
 // the keys in flight stay in flight.
 // Registers are the limit (128 for the scores, 64 for the queries during step 1): what depends on the
 // thread is derived again after step 1 from opaque copies instead of being kept across it.
-// chunks of 64 keys per workgroup and pair
-__host__ __device__ constexpr int fused_chunks(int qh) { return qh == 1 ? 16 : 8; }
+// chunks of 64 keys per workgroup and pair: 16 for up to 64 queries, 8 for up to 128; 32 when a wave holds two
+// groups of sixteen queries (nq) instead of four
+__host__ __device__ constexpr int fused_chunks(int qh, int nq = 4) { return qh == 1 ? 16 * (4 / nq) : 8; }
 constexpr int kFusedSteps = 8;
 constexpr int kFusedThreads = 512;
 
@@ -1179,18 +1182,24 @@ __global__ __launch_bounds__(256) void zero_words_kernel(unsigned* __restrict__ 
 // Eight waves, one workgroup per CU, eight steps per workgroup and pair.  Up to 64 queries (QH = 1, KH = 2):
 // a step is two chunks of 64 keys, waves 0-3 take (and load) the first, waves 4-7 the second.  Up to 128
 // queries (QH = 2, KH = 1): a step is one chunk, waves 4-7 hold queries 64-127, waves 0-3 load.
-template <int DT, int KS, bool CAUSAL, int MODE, int QH>
+// NQ: groups of sixteen queries a wave holds (4; 2 for at most 32 queries: the registers then hold the scores of
+// twice as many keys per pair, and the time between two sweeps is spread over that many.  One group and four
+// times the keys was built as well and was slower than two: 1568 against 1499 us on 64 x 32 pairs of 16384 keys).
+template <int DT, int KS, bool CAUSAL, int MODE, int QH, int NQ = 4>
 __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Params p) {
-  constexpr int KG = kFusedSteps;
+  static_assert(NQ == 4 || (QH == 1 && NQ == 2), "fewer query groups only with one query half");
+  constexpr int KG = kFusedSteps * (4 / NQ);     // steps per pair
   constexpr int KH = 3 - QH;                     // chunks per step
   constexpr int NS = (QH == 1) ? 8 : 6;          // ring stages (chunks): 130 KiB or 98 KiB for 256-byte rows
   using Rg = Ring<KS, NS>;                       // four loads of 1 KiB per loading wave and chunk for 256-byte rows
   constexpr int kQBytes = QH * Rg::kRows;        // the queries of a pair, staged like a chunk of keys per 64 rows
   constexpr int kNumThreads = kFusedThreads;
-  constexpr int kRowsWg = 64 * QH;               // query rows a workgroup holds
-  constexpr int kItemKeys = KG * KH * kChunk;
+  constexpr int kRowsWg = 16 * NQ * QH;          // query rows a workgroup holds
+  constexpr int kItemKeys = KG * KH * kChunk;    // keys of a workgroup per pair
+  constexpr int kBatchKeys = kFusedSteps * KH * kChunk;   // finished columns leave eight steps at a time
+  constexpr int kBatches = KG / kFusedSteps;
   constexpr int kRes = (MODE == kModeBoth) ? 2 : 1;
-  constexpr int kObufFloats = QH * kRes * kItemKeys;
+  constexpr int kObufFloats = QH * kRes * kBatchKeys;
   constexpr int kRedFloats = 8 * 64;
   // waves per row that share the merge of the team's partial values (half of them when two results are
   // buffered for 1024 keys: the LDS is full)
@@ -1289,10 +1298,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
   };
   int cons_chunk = 0;       // number of the next chunk to be computed (its stage: cons_chunk % NS)
 
-  int qrows[4];
-#pragma unroll
-  for (int g = 0; g < 4; ++g) qrows[g] = 64 * qh + 16 * g;
-  u32x4 qf[4][KS];
+  u32x4 qf[NQ][KS];
   // The queries of a pair go from memory to LDS like a chunk of keys (64 rows per stage-like tile, same
   // swizzle), long before they are needed, and from there into the registers when the pair's sweep starts:
   // no wave ever waits for them, and they take no registers between two sweeps.  Waves 0-3 load.
@@ -1317,7 +1323,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
   };
   auto read_queries = [&]() {
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
+    for (int g = 0; g < NQ; ++g)
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) qf[g][ks] = rg.frag(qlds + qh * Rg::kRows, g >> 1, g & 1, ks);
   };
@@ -1331,7 +1337,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
   // Register (g, r) of a lane is query 64*qh + 16g + qrow + r against the lane's key.  It takes part iff
   // the query exists and may see the key: 16g + r in [first, mlim).
   const int mlim0 = p.M - 64 * qh - qrow0;
-  const bool ragged_rows = p.M < 64 * (qh + 1);
+  const bool ragged_rows = p.M < 16 * NQ * (qh + 1);
   constexpr int kRowWaves = 8 / QH;   // row tid (tid < kRowsWg) is held by all eight waves, or by 0-3 / 4-7 for rows below / from 64
 
   for (int it = 0; it < rounds; ++it) {
@@ -1339,8 +1345,8 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     // What the registers keep per score: for column sums 2^score (step 4 is then one multiply-add per score),
     // otherwise, or when a row's sum of 2^score is unusable, the score itself.  In the second case of a sum
     // the scores are gone by the time it shows, and the keys of the pair are streamed once more.
-    f32x4 sc[KG][4];
-    f32x4 rs[4];   // per row (register) and key (lane): sum of 2^score over the steps
+    f32x4 sc[KG][NQ];
+    f32x4 rs[NQ];   // per row (register) and key (lane): sum of 2^score over the steps
     float my_lse = kNegInf;   // of row tid over this workgroup's keys, for tid < kRowsWg
     // Steps 1 and the first half of 2, in two forms (KEEP: the registers end up holding the scores).  Returns
     // whether some row's sum of 2^score is unusable.
@@ -1348,7 +1354,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     constexpr bool KEEP = decltype(keep_tag)::value;
     if (KEEP) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int g = 0; g < NQ; ++g) rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
     }
     {
     const int tid = tid0, lane = lane0, qrow = qrow0, mlim = mlim0;
@@ -1366,21 +1372,25 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
       if (j == 1 && it + 1 < rounds) stage_queries(bh + T);   // every wave has read this pair's by now
       const char* lds = stage_of(cons_chunk + j * KH + kh);
 #pragma unroll
-      for (int g = 0; g < 4; ++g) sc[j][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int g = 0; g < NQ; ++g) sc[j][g] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const u32x4 kfrag = rg.frag(lds, wq >> 1, wq & 1, ks);
 #pragma unroll
-        for (int g = 0; g < 4; ++g) sc[j][g] = mma<DT>(qf[g][ks], kfrag, sc[j][g]);
+        for (int g = 0; g < NQ; ++g) sc[j][g] = mma<DT>(qf[g][ks], kfrag, sc[j][g]);
       }
       const int kbase = (c0a + j * KH + kh) * kChunk;
       const int key = kbase + 16 * wq + (lane & 15);
-      const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * qh);
+      // Rows past M are rows of zeros: their scores are 0 and their 2^score is 1, which nothing downstream uses
+      // (their factor in step 4 is 0), so the fast form of the sweep does not hide them.  Only a key with a
+      // non-finite element makes them NaN; the row threads below look for that and ask for the second sweep,
+      // which hides them as every sweep that keeps scores does.
+      const bool need_mask = (KEEP && ragged_rows) || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * qh);
       if (need_mask) {
         int first = CAUSAL ? key - p.c - 64 * qh - qrow : -(1 << 30);
         if (key >= p.N) first = 1 << 30;
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < NQ; ++g)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int o = 16 * g + r;
@@ -1388,16 +1398,16 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
           }
       } else {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) sc[j][g] *= p.scale2;
+        for (int g = 0; g < NQ; ++g) sc[j][g] *= p.scale2;
       }
       if (KEEP) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < NQ; ++g)
 #pragma unroll
           for (int r = 0; r < 4; ++r) rs[g][r] += fast_exp2(sc[j][g][r]);
       } else {   // (the row sums are taken after the loop: sixteen registers less while the queries are held)
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < NQ; ++g)
 #pragma unroll
           for (int r = 0; r < 4; ++r) sc[j][g][r] = fast_exp2(sc[j][g][r]);
       }
@@ -1406,7 +1416,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     }
     if (!KEEP) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int g = 0; g < NQ; ++g) {
         rs[g] = sc[0][g];
 #pragma unroll
         for (int j = 1; j < KG; ++j) rs[g] += sc[j][g];
@@ -1424,7 +1434,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     // came; they are good unless a sum left fp32's comfortable range (or a row saw no key at all), and then
     // the scores, still in registers, are reduced again the exact way: row maximum first.
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
+    for (int g = 0; g < NQ; ++g) {
 #pragma unroll
       for (int r = 0; r < 4; ++r) rs[g][r] = row16_reduce<false>(rs[g][r]);
       if ((lane & 15) == 0) *reinterpret_cast<f32x4*>(red + wave * 64 + 16 * g + qrow) = rs[g];
@@ -1439,6 +1449,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
       // (the lse of all keys is at least this one) neither overflows nor loses anything above 2^-26
       const bool good = (l >= 8.6736174e-19f) && (l < 1.2676506e30f);
       if (!good && tid < p.M) flag[0] = 1;   // (written by whoever finds a bad row; thread 0 resets it below)
+      if (!KEEP && tid >= p.M && !(l < kPosInf)) flag[0] = 1;   // a row of zeros met a non-finite key
       if (tid == 0) flag[1] = 1;
     }
     lds_barrier();
@@ -1470,9 +1481,9 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     const int mlim = p.M - 64 * qh - qrow;
     const float* const red_row = red + (QH == 2 ? (tid >> 6) * (kWaves * 64) : 0) + (tid & 63);
     if (bad_sum) {
-      f32x4 rm[4];
+      f32x4 rm[NQ];
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int g = 0; g < NQ; ++g) {
         rm[g] = sc[0][g];
 #pragma unroll
         for (int j = 1; j < KG; ++j)
@@ -1491,7 +1502,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
       }
       lds_barrier();
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int g = 0; g < NQ; ++g) {
         const f32x4 ref = *reinterpret_cast<const f32x4*>(rowv + 64 * qh + 16 * g + qrow);
         rs[g] = (f32x4){0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -1526,6 +1537,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     // for the next pair return before these loads do; they were requested during the last steps above.)
     if (wave / QH < kMergeWaves) {
       const int rgroup = wave % QH, sub = wave / QH;
+      const bool row_here = 64 * rgroup + lane < kRowsWg;   // (fewer than 64 rows per workgroup with NQ < 4)
       const unsigned long long* mine = slots + 64 * rgroup + lane;
       float m = kNegInf, acc = 0.f;
       bool nan = false, ok = true;
@@ -1537,7 +1549,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
 #pragma unroll
           for (int i = 0; i < kBatch; ++i) {
             const int sidx = s0 + i * kMergeWaves;
-            w[i] = (sidx < S) ? __hip_atomic_load(mine + (int64_t)sidx * kRowsWg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+            w[i] = (sidx < S && row_here) ? __hip_atomic_load(mine + (int64_t)sidx * kRowsWg, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
                               : (((unsigned long long)round_no << 32) | 0xff800000u);   // -inf: adds nothing
           }
 #pragma unroll
@@ -1571,8 +1583,10 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
         flag[1] = 0;
       }
       // a NaN partial (fmaxf drops it) makes the row's lse NaN
-      mrg[(sub * kRowsWg + 64 * rgroup + lane) * 2] = nan ? __builtin_nanf("") : m;
-      mrg[(sub * kRowsWg + 64 * rgroup + lane) * 2 + 1] = acc;
+      if (row_here) {
+        mrg[(sub * kRowsWg + 64 * rgroup + lane) * 2] = nan ? __builtin_nanf("") : m;
+        mrg[(sub * kRowsWg + 64 * rgroup + lane) * 2 + 1] = acc;
+      }
     }
     lds_barrier();
     if (tid < kRowsWg) {
@@ -1605,19 +1619,22 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
     if (tid == 0) flag[0] = 0;
     if (!met) spin_limit = min(spin_limit, 64);   // the call has failed: later waits of this workgroup are short
     // 4. probabilities, reduced down the rows
-    f32x4 nl[4];
+    f32x4 nl[NQ];
 #pragma unroll
-    for (int g = 0; g < 4; ++g) nl[g] = *reinterpret_cast<const f32x4*>(rowv + 64 * qh + 16 * g + qrow);
-    float* const osum = obuf + qh * (kRes * kItemKeys);
-    float* const omax = osum + (MODE == kModeBoth ? kItemKeys : 0);
+    for (int g = 0; g < NQ; ++g) nl[g] = *reinterpret_cast<const f32x4*>(rowv + 64 * qh + 16 * g + qrow);
+    float* const osum = obuf + qh * (kRes * kBatchKeys);
+    float* const omax = osum + (MODE == kModeBoth ? kBatchKeys : 0);
     int c0b = c0;
     asm volatile("" : "+s"(c0b));
-    float vs[KG], vm[KG];   // per step: the lane's key, reduced over the lane's sixteen queries
 #pragma unroll
-    for (int j = 0; j < KG; ++j) {
+    for (int bt = 0; bt < kBatches; ++bt) {   // eight steps at a time through the column buffer
+    float vs[kFusedSteps], vm[kFusedSteps];   // per step: the lane's key, reduced over the lane's queries
+#pragma unroll
+    for (int jj = 0; jj < kFusedSteps; ++jj) {
+      const int j = bt * kFusedSteps + jj;
       const int kbase = (c0b + j * KH + kh) * kChunk;
       const int key = kbase + 16 * wq + (lane & 15);
-      const bool need_mask = ragged_rows || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * qh);
+      const bool need_mask = (keep_scores && ragged_rows) || kbase + kChunk > p.N || (CAUSAL && kbase + kChunk - 1 > p.c + 64 * qh);
       f32x4 part = {0.f, 0.f, 0.f, 0.f};   // four independent chains
       float vmax = kNegInf;
       if (MODE == kModeSum && !keep_scores) {   // the registers hold 2^score, nl holds 2^-lse
@@ -1625,7 +1642,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
           int first = CAUSAL ? key - p.c - 64 * qh - qrow : -(1 << 30);
           if (key >= p.N) first = 1 << 30;
 #pragma unroll
-          for (int g = 0; g < 4; ++g)
+          for (int g = 0; g < NQ; ++g)
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const int o = 16 * g + r;
@@ -1633,7 +1650,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
             }
         } else {
 #pragma unroll
-          for (int g = 0; g < 4; ++g)
+          for (int g = 0; g < NQ; ++g)
 #pragma unroll
             for (int r = 0; r < 4; ++r) part[r] = fmaf(sc[j][g][r], nl[g][r], part[r]);
         }
@@ -1641,7 +1658,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
         int first = CAUSAL ? key - p.c - 64 * qh - qrow : -(1 << 30);
         if (key >= p.N) first = 1 << 30;
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < NQ; ++g)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const int o = 16 * g + r;
@@ -1651,7 +1668,7 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
           }
       } else {
 #pragma unroll
-        for (int g = 0; g < 4; ++g)
+        for (int g = 0; g < NQ; ++g)
 #pragma unroll
           for (int r = 0; r < 4; ++r) {
             const float x = sc[j][g][r] + nl[g][r];
@@ -1659,53 +1676,56 @@ __global__ __launch_bounds__(kFusedThreads, 2) void col_fused_kernel(const Param
             if (MODE != kModeMax) part[r] += fast_exp2(x);
           }
       }
-      vs[j] = (part[0] + part[1]) + (part[2] + part[3]);
-      vm[j] = vmax;
+      vs[jj] = (part[0] + part[1]) + (part[2] + part[3]);
+      vm[jj] = vmax;
     }
     // the four lane groups hold different queries of the same key: two exchanges, all steps at once
     if (MODE != kModeMax) {
-      float o[KG];
+      float o[kFusedSteps];
 #pragma unroll
-      for (int j = 0; j < KG; ++j) o[j] = __shfl_xor(vs[j], 16);
+      for (int j = 0; j < kFusedSteps; ++j) o[j] = __shfl_xor(vs[j], 16);
 #pragma unroll
-      for (int j = 0; j < KG; ++j) vs[j] += o[j];
+      for (int j = 0; j < kFusedSteps; ++j) vs[j] += o[j];
 #pragma unroll
-      for (int j = 0; j < KG; ++j) o[j] = __shfl_xor(vs[j], 32);
+      for (int j = 0; j < kFusedSteps; ++j) o[j] = __shfl_xor(vs[j], 32);
       if (lane < 16) {
 #pragma unroll
-        for (int j = 0; j < KG; ++j) osum[(j * KH + kh) * kChunk + 16 * wq + lane] = vs[j] + o[j];
+        for (int j = 0; j < kFusedSteps; ++j) osum[(j * KH + kh) * kChunk + 16 * wq + lane] = vs[j] + o[j];
       }
     }
     if (MODE != kModeSum) {
-      float o[KG];
+      float o[kFusedSteps];
 #pragma unroll
-      for (int j = 0; j < KG; ++j) o[j] = __shfl_xor(vm[j], 16);
+      for (int j = 0; j < kFusedSteps; ++j) o[j] = __shfl_xor(vm[j], 16);
 #pragma unroll
-      for (int j = 0; j < KG; ++j) vm[j] = fmaxf(vm[j], o[j]);
+      for (int j = 0; j < kFusedSteps; ++j) vm[j] = fmaxf(vm[j], o[j]);
 #pragma unroll
-      for (int j = 0; j < KG; ++j) o[j] = __shfl_xor(vm[j], 32);
+      for (int j = 0; j < kFusedSteps; ++j) o[j] = __shfl_xor(vm[j], 32);
       if (lane < 16) {
 #pragma unroll
-        for (int j = 0; j < KG; ++j) omax[(j * KH + kh) * kChunk + 16 * wq + lane] = fast_exp2(fmaxf(vm[j], o[j]));
+        for (int j = 0; j < kFusedSteps; ++j) omax[(j * KH + kh) * kChunk + 16 * wq + lane] = fast_exp2(fmaxf(vm[j], o[j]));
       }
     }
     lds_barrier();
     void* const out_max = (MODE == kModeBoth) ? p.out2 : p.out;
     const float poison = __builtin_nanf("");
-    for (int i = tid; i < kItemKeys; i += kNumThreads) {
-      if (key0 + i < keys_end) {
+    const int bkey0 = key0 + bt * kBatchKeys;
+    for (int i = tid; i < kBatchKeys; i += kNumThreads) {
+      if (bkey0 + i < keys_end) {
         if (MODE != kModeMax) {
           float v = obuf[i];
-          if (QH == 2) v += obuf[kRes * kItemKeys + i];
-          store_column(p, p.out, true, bh, key0 + i, met ? v : poison);
+          if (QH == 2) v += obuf[kRes * kBatchKeys + i];
+          store_column(p, p.out, true, bh, bkey0 + i, met ? v : poison);
         }
         if (MODE != kModeSum) {
-          const float* om = obuf + (MODE == kModeBoth ? kItemKeys : 0);
+          const float* om = obuf + (MODE == kModeBoth ? kBatchKeys : 0);
           float v = om[i];
-          if (QH == 2) v = fmaxf(v, om[kRes * kItemKeys + i]);
-          store_column(p, out_max, false, bh, key0 + i, met ? v : poison);
+          if (QH == 2) v = fmaxf(v, om[kRes * kBatchKeys + i]);
+          store_column(p, out_max, false, bh, bkey0 + i, met ? v : poison);
         }
       }
+    }
+    if (bt + 1 < kBatches) lds_barrier();   // the next batch writes the buffer again
     }
     // the next writers of obuf, red, rowv and flag are behind the ring barriers of the next pair
   }
@@ -2303,6 +2323,7 @@ int row_splits(int B, int H, int M, int N, int ksteps) {
 constexpr int kFusedMinChunks = 16;   // 1024 keys
 struct FusedPlan {
   int qh;       // 1: 64 query rows per workgroup and 1024 keys per pair, 2: 128 rows and 512 keys
+  int nq;       // groups of sixteen queries per wave: 4, or 2 (at most 32 queries) with 2048 keys per pair
   int splits, teams;
   int64_t part_at, sync_at;   // where the partial row values and the counters start in the workspace, in floats
   int64_t floats;             // workspace size
@@ -2313,11 +2334,28 @@ bool fused_shape(int64_t bh, int M, int N, FusedPlan& f) {
   if (M > 2 * 64 || nchunks < kFusedMinChunks) return false;
   f.qh = M > 64 ? 2 : 1;
   const int cap = chip_cus();   // one workgroup per CU
-  const int64_t splits = (nchunks + fused_chunks(f.qh) - 1) / fused_chunks(f.qh);
-  if (splits > cap) return false;
-  f.splits = (int)splits;
-  const int64_t teams = cap / splits;
-  f.teams = (int)(teams < bh ? teams : bh);
+  // With at most 32 queries a workgroup can keep the scores of 2048 keys of a pair, which spreads the time
+  // between two sweeps over twice the keys, but it leaves half the workgroups per pair.  The choice is the
+  // one with the least estimated time: rounds x (0.56 us per chunk + 4.5 us between sweeps).
+  double best = 0.0;
+  f.nq = 0;
+  for (int nq = 4; nq >= 2; nq /= 2) {
+    if (nq < 4 && (f.qh != 1 || M > 16 * nq)) continue;
+    const int chunks = fused_chunks(f.qh, nq);
+    const int64_t splits = (nchunks + chunks - 1) / chunks;
+    if (splits > cap) continue;
+    const int64_t teams = (cap / splits) < bh ? (cap / splits) : bh;
+    const int64_t rounds = (bh + teams - 1) / teams;
+    const int64_t swept = nchunks < chunks ? nchunks : chunks;
+    const double cost = (double)rounds * (0.56 * (double)swept + 4.5);
+    if (f.nq == 0 || cost < best) {
+      best = cost;
+      f.nq = nq;
+      f.splits = (int)splits;
+      f.teams = (int)teams;
+    }
+  }
+  if (f.nq == 0) return false;
   f.part_at = (bh * M + 63) / 64 * 64;
   f.sync_at = f.part_at + 2 * (2ll * cap * 64 * f.qh);   // two sets of one 64-bit slot per row and workgroup
   f.floats = f.sync_at + 32;
@@ -2397,37 +2435,39 @@ bool fits_per_cu(K kernel, int threads, int want) {
   return n >= want;
 }
 
-template <int DT, int KS, int MODE, int QH>
+template <int DT, int KS, int MODE, int QH, int NQ = 4>
 void launch_col_fused_mode(const Params& p, bool causal, hipStream_t s) {
   const dim3 grid(p.total), block(kFusedThreads);
   static int fits[2] = {-1, -1};   // asked once per kernel (the answer depends on its registers and LDS, not on the device of a kind)
   int f = __atomic_load_n(&fits[causal], __ATOMIC_RELAXED);
   if (f < 0) {
-    f = causal ? fits_per_cu(col_fused_kernel<DT, KS, true, MODE, QH>, kFusedThreads, 1)
-               : fits_per_cu(col_fused_kernel<DT, KS, false, MODE, QH>, kFusedThreads, 1);
+    f = causal ? fits_per_cu(col_fused_kernel<DT, KS, true, MODE, QH, NQ>, kFusedThreads, 1)
+               : fits_per_cu(col_fused_kernel<DT, KS, false, MODE, QH, NQ>, kFusedThreads, 1);
     __atomic_store_n(&fits[causal], f, __ATOMIC_RELAXED);
   }
   if (!f) {
     fcr_detail::fused_refused = true;
     return;
   }
-  if (causal) hipLaunchKernelGGL((col_fused_kernel<DT, KS, true, MODE, QH>), grid, block, 0, s, p);
-  else hipLaunchKernelGGL((col_fused_kernel<DT, KS, false, MODE, QH>), grid, block, 0, s, p);
+  if (causal) hipLaunchKernelGGL((col_fused_kernel<DT, KS, true, MODE, QH, NQ>), grid, block, 0, s, p);
+  else hipLaunchKernelGGL((col_fused_kernel<DT, KS, false, MODE, QH, NQ>), grid, block, 0, s, p);
 }
 
-// mode: kModeSum, kModeMax or kModeBoth, + 4 for more than 64 queries
+template <int DT, int KS, int QH, int NQ>
+void launch_col_fused_groups(const Params& p, bool causal, int m, hipStream_t s) {
+  if (m == kModeSum) launch_col_fused_mode<DT, KS, kModeSum, QH, NQ>(p, causal, s);
+  else if (m == kModeMax) launch_col_fused_mode<DT, KS, kModeMax, QH, NQ>(p, causal, s);
+  else launch_col_fused_mode<DT, KS, kModeBoth, QH, NQ>(p, causal, s);
+}
+
+// mode: kModeSum, kModeMax or kModeBoth, + 4 for more than 64 queries, + 8 for two groups of sixteen queries
+// per wave
 template <int DT, int KS>
 void launch_col_fused(const Params& p, bool causal, int mode, hipStream_t s) {
   const int m = mode & 3;
-  if (mode & 4) {
-    if (m == kModeSum) launch_col_fused_mode<DT, KS, kModeSum, 2>(p, causal, s);
-    else if (m == kModeMax) launch_col_fused_mode<DT, KS, kModeMax, 2>(p, causal, s);
-    else launch_col_fused_mode<DT, KS, kModeBoth, 2>(p, causal, s);
-  } else {
-    if (m == kModeSum) launch_col_fused_mode<DT, KS, kModeSum, 1>(p, causal, s);
-    else if (m == kModeMax) launch_col_fused_mode<DT, KS, kModeMax, 1>(p, causal, s);
-    else launch_col_fused_mode<DT, KS, kModeBoth, 1>(p, causal, s);
-  }
+  if (mode & 4) launch_col_fused_groups<DT, KS, 2, 4>(p, causal, m, s);
+  else if (mode & 8) launch_col_fused_groups<DT, KS, 1, 2>(p, causal, m, s);
+  else launch_col_fused_groups<DT, KS, 1, 4>(p, causal, m, s);
 }
 
 template <int DT, int KS>
@@ -2481,14 +2521,23 @@ void launch_col(const Params& p, bool causal, int mode, hipStream_t s) {
   void fcr_detail::NAME(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) { \
     if (which == 0) { FCR_DISPATCH_KS(DT, ksteps, FCR_CALL_LSE) }                                        \
     else if (which == 1) { FCR_DISPATCH_KS(DT, ksteps, FCR_CALL_COL) }                                   \
-    else if (which == 2) { FCR_DISPATCH_KS4(DT, ksteps, FCR_CALL_COL_SMALL) }                            \
-    else { FCR_DISPATCH_KS4(DT, ksteps, FCR_CALL_COL_FUSED) }                                            \
+    else { FCR_DISPATCH_KS4(DT, ksteps, FCR_CALL_COL_SMALL) }                                            \
   }
 #if FCR_HAS(1)
 FCR_SWEEPS_16BIT(sweeps_f16, FCR_DTYPE_F16)
 #endif
 #if FCR_HAS(2)
 FCR_SWEEPS_16BIT(sweeps_bf16, FCR_DTYPE_BF16)
+#endif
+#if FCR_HAS(7)
+void fcr_detail::sweeps_f16_single(const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
+  FCR_DISPATCH_KS4(FCR_DTYPE_F16, ksteps, FCR_CALL_COL_FUSED)
+}
+#endif
+#if FCR_HAS(8)
+void fcr_detail::sweeps_bf16_single(const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
+  FCR_DISPATCH_KS4(FCR_DTYPE_BF16, ksteps, FCR_CALL_COL_FUSED)
+}
 #endif
 #if FCR_HAS(3)
 void fcr_detail::sweeps_f32(int which, const Params& p, int ksteps, bool causal, int mode, hipStream_t s) {
@@ -2527,6 +2576,11 @@ void launch_sweeps(int dtype, int which, const Params& p, int ksteps, bool causa
   if (zero_words > 0)
     hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((zero_words + 255) / 256)), dim3(256), 0, s, zero, zero_words);
   const bool long_rows = ksteps > kMaxKSteps;
+  if (which == 3) {   // the single sweep: 16-bit elements, rows of at most 256 bytes
+    if (dtype == FCR_DTYPE_F16) fcr_detail::sweeps_f16_single(p, ksteps, causal, mode, s);
+    else fcr_detail::sweeps_bf16_single(p, ksteps, causal, mode, s);
+    return;
+  }
   if (dtype == FCR_DTYPE_F16) (long_rows ? fcr_detail::sweeps_f16_long_rows : fcr_detail::sweeps_f16)(which, p, ksteps, causal, mode, s);
   else if (dtype == FCR_DTYPE_BF16) (long_rows ? fcr_detail::sweeps_bf16_long_rows : fcr_detail::sweeps_bf16)(which, p, ksteps, causal, mode, s);
   else (long_rows ? fcr_detail::sweeps_f32_long_rows : fcr_detail::sweeps_f32)(which, p, ksteps, causal, mode, s);
@@ -2831,8 +2885,8 @@ int whole_call(const void* q, const void* k, void* out, const ResultSpec& res, f
     const int words = (int)(f.floats - f.part_at);   // the slots and the error word start at zero
     fcr_detail::fused_refused = false;
     SweepOrder* const order = (ws_bytes == 0) ? order_begin(s) : nullptr;
-    launch_sweeps(dtype, 3, p, ksteps, causal != 0, mode | (f.qh == 2 ? 4 : 0), s, reinterpret_cast<unsigned*>(p.part),
-                  words);
+    launch_sweeps(dtype, 3, p, ksteps, causal != 0, mode | (f.qh == 2 ? 4 : 0) | (f.nq == 2 ? 8 : 0), s,
+                  reinterpret_cast<unsigned*>(p.part), words);
     const int lrc = fcr_detail::fused_refused ? 0 : launched("col_fused_kernel");
     order_end(order, s, !fcr_detail::fused_refused && lrc == 0);
     if (!fcr_detail::fused_refused) return lrc;

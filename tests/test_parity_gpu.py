@@ -359,6 +359,11 @@ def _c_abi_colreduce(q, k, red, causal, scale=None):
     (2, 7, 17, 2100, 16),      # rows of 32 bytes
     (1, 1, 1, 70000, 128),     # one query, 69 workgroups on one pair
     (40, 16, 64, 2048, 32),    # 640 pairs for 128 teams: five rounds per workgroup
+    (40, 16, 16, 8192, 64),    # at most 32 queries: two groups of queries per wave, 2048 keys per workgroup and pair
+    (8, 32, 32, 8192, 128),    # the same with all 32 rows
+    (64, 8, 7, 4100, 128),     # a ragged third workgroup
+    (300, 4, 9, 1500, 32),     # a single workgroup per pair sweeping less than its share
+    (3, 5, 20, 9000, 72),      # ragged everything
 ])
 def test_single_sweep(b, h, m, n, d, causal, dtype):
     """At most 128 queries against at least 1024 keys: one sweep over the keys computes the row statistics
@@ -436,6 +441,26 @@ def test_single_sweep_nan_and_inf_inputs(causal):
         if causal:
             assert ok[0, 0].any() and ok[0, 1].any()
         check(got[ok], want[ok], red, f"single sweep, columns no NaN row sees, causal={causal}")
+
+
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("m", [3, 20, 40, 100])
+def test_single_sweep_rows_of_padding_meet_a_non_finite_key(m, causal):
+    """Fewer queries than a workgroup holds rows for: the rows of padding are rows of zeros, which the fast form
+    of the sweep leaves in place.  A key with an infinite element turns their scores into NaN (0 * inf); the
+    sweep notices and hides them the slow way.  Here every real query is positive where the key is -inf, so
+    the key's scores are -inf, its column is exactly 0 and every other column is untouched."""
+    b, h, n, d = 2, 3, 3000, 64
+    q, k = _inputs.randn_pair(b, h, m, n, d, seed=91 + m)
+    q, k = q.half().clone(), k.half().clone()
+    q[..., 7] = q[..., 7].abs() + 0.5
+    k[0, 1, 1234, 7] = float("-inf")
+    k[1, 2, n - 1, 7] = float("-inf")
+    for red in REDUCTIONS:
+        got = fca.flash_colreduce(q.cuda(), k.cuda(), red, is_causal=causal, out_dtype=torch.float32).cpu()
+        assert not torch.isnan(got).any(), red
+        assert got[0, 1, 1234] == 0 and got[1, 2, n - 1] == 0
+        check(got, colreduce_ref(q, k, red, causal), red, f"padding rows m{m} {red}")
 
 
 def test_single_sweep_bounded_wait():
